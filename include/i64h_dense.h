@@ -27,8 +27,13 @@ int i64h_device_check(void);
  * exact = 1: W is widened to fp32 while it is staged, products on v_mfma_f32_16x16x4_f32: true 32-bit arithmetic.
  * epilogue: I64H_EPI_STORE; I64H_EPI_GELU_MUL: gelu_tanh(A W^T) * (A W2^T) with W2 = W + N * K (gate rows, then up rows);
  *   I64H_EPI_MUL_SIGMOID: * sigmoid(E[b][m, n]) (E fp32, row stride lde, batch stride e_batch);
- *   I64H_EPI_SOFTCAP: cap * tanh(. / cap);  I64H_EPI_GELU_ERF: 0.5 v (1 + erf(v / sqrt 2));  I64H_EPI_SCALE: v * scale.
- *   bias (may be NULL; fp32 [N], batch stride bias_batch) is added to the sum before any epilogue but I64H_EPI_GELU_MUL.
+ *   I64H_EPI_SOFTCAP: cap * tanh(. / cap);  I64H_EPI_GELU_ERF: 0.5 v (1 + erf(v / sqrt 2));  I64H_EPI_SCALE: v * scale;
+ *   I64H_EPI_SILU_MUL: silu(A W^T) * (A W2^T), laid out as I64H_EPI_GELU_MUL;
+ *   I64H_EPI_XIELU: v > 0 ? act_a v^2 + v / 2 : act_b (exp(v) - 1 - v) + v / 2  (the caller passes act_a = softplus(p), act_b = 1/2 + softplus(q)).
+ *   bias (may be NULL; fp32 [N], batch stride bias_batch) is added to the sum before any epilogue but the two gate / up ones.
+ * group_off (may be NULL; device int32 [batch + 1], ascending): batch b takes the rows [group_off[b], group_off[b + 1]) of a_rows
+ *   (of A itself without a_rows) and of C instead of all M rows; M is then the most rows any batch may have (it sizes the launch,
+ *   workgroups past a batch's rows leave at once), and the launch needs no count on the host.  Such launches take the 64 x 64 tile form.
  * Any M, N, K >= 1; 16-byte loads are used where strides and addresses allow, element loads otherwise.
  * Launches with M <= I64H_SKINNY_ROWS take a weight-streaming form (one wave per output column group). */
 #define I64H_EPI_STORE 0
@@ -37,6 +42,8 @@ int i64h_device_check(void);
 #define I64H_EPI_SOFTCAP 3
 #define I64H_EPI_GELU_ERF 4
 #define I64H_EPI_SCALE 5
+#define I64H_EPI_SILU_MUL 6
+#define I64H_EPI_XIELU 7
 #define I64H_SKINNY_ROWS 8
 typedef struct {
     const float* A;
@@ -57,6 +64,8 @@ typedef struct {
     const float* bias;
     int64_t bias_batch;
     float scale;
+    float act_a, act_b;
+    const int32_t* group_off;
 } i64h_linear;
 int i64h_linear_run(const i64h_linear* d, void* stream);
 
@@ -168,7 +177,8 @@ int i64h_latent_attn(const i64h_latent_attn_args* d, void* stream);
  * out[c][t, :] = table[ids[t]] + bigram[row(t)] for c < copies (out fp32 [copies, n, W]);  row(t) = buckets at position 0, else
  * (previous * mul_prev + ids[t] * mul_cur) mod buckets, previous = the token of the row before in the same sequence, or
  * prev_token[slot] (the last token of the sequence's earlier steps).  A second launch stores every sequence's last token of
- * this step in prev_token.  bigram == NULL: the token embedding alone.  Tables bf16. */
+ * this step in prev_token.  bigram == NULL: the token embedding alone.  pos_table (may be NULL; bf16 [pos_rows, W]): the row of the
+ * token's position is added (positions past the table take its last row; callers bound positions by pos_rows).  Tables bf16. */
 typedef struct {
     const int64_t* ids;
     const int32_t* positions;
@@ -182,12 +192,15 @@ typedef struct {
     float* out;
     int32_t copies;
     int64_t n;
+    const void* pos_table;
+    int64_t pos_rows;
 } i64h_embed_bigram_args;
 int i64h_embed_bigram(const i64h_embed_bigram_args* d, void* stream);
 
 /* ---- multi-stream residual (hyper-connections) with the next sublayer's RMS norm -------------------------------------------------
  * streams fp32 [S, n, W], updated in place, one workgroup per row:
- *   write (y != NULL):  v = y2 ? 0.5 * (rms(y) * yn_w + rms(y2) * y2n_w) : y      (rms over the W columns with y_eps; weights [W])
+ *   write (y != NULL):  v = y2 ? 0.5 * (rms(y) * yn_w + rms(y2) * y2n_w) : (yn_w ? rms(y) * yn_w : y)
+ *                       (rms over the W columns with y_eps; weights [W]; a single normed result is the post-norm of a sandwich layer)
  *                       new_t = sum_s mix[s * S + t] * old_s + out_w[t] * v          (mix == NULL: new_t = old_t + out_w[t] * v)
  *   read  (h != NULL):  u = sum_s in_w[s] * x_s  (in_w == NULL: the plain sum);  h = u / sqrt(mean(u^2) + eps) * norm_w[c % norm_w_len]
  * rows (may be NULL, read only launches): h[m] is computed from row rows[m] of the streams (the rows whose logits are wanted). */
@@ -219,7 +232,8 @@ int i64h_streams_step(const i64h_streams_args* d, void* stream);
  * out[t, c] = silu(bias[c] + sum_k w[c, k] * in(t, taps - 1 - k)),  in(t, d) = the input of channel c d positions before row t:
  * zero before position 0, a row of this step where the sequence has one there, else the carried inputs state fp32
  * [slots, taps - 1, channels] (the last taps - 1 inputs of the sequence's earlier steps, oldest first).  Inputs are the columns
- * [off, off + channels) of P.  A second launch stores the new carried inputs.  w fp32 [channels, taps]. */
+ * [off, off + channels) of P.  A second launch stores the new carried inputs.  w fp32 [channels, taps].
+ * mode 1: out[t, c] = in(t, 0) + bias[c] + sum_k ... without the activation (a convolution added to its own input). */
 typedef struct {
     const float* P;
     int64_t ldp;
@@ -232,6 +246,7 @@ typedef struct {
     float* out;
     int64_t ldo;
     int64_t n;
+    int32_t mode;
 } i64h_causal_conv_args;
 int i64h_causal_conv(const i64h_causal_conv_args* d, void* stream);
 
@@ -350,9 +365,105 @@ typedef struct {
                             prompts), 0 / 2 a wave per token and 16 query heads of one key head (rows that are one per sequence) */
     int32_t splits;      /* mode 0 / 2: every token's keys are dealt to this many waves and merged by a second launch */
     float* workspace;    /* i64h_kattn_workspace_floats(n, heads, kv_heads, dim, splits) floats when splits > 1 */
+    int32_t vdim;        /* > 0: keys and values are separate (see i64h_kv_prep): a cached row holds per key head [vdim values | dim key values], Q is
+                            [n, heads, vdim + dim] with the query in the last dim columns of a head, out [n, heads, vdim], kscale may be NULL;
+                            the workspace is then i64h_kattn_workspace_floats(n, heads, kv_heads, vdim, splits) floats */
 } i64h_kattn_args;
 int64_t i64h_kattn_workspace_floats(int64_t n, int32_t heads, int32_t kv_heads, int32_t dim, int32_t splits);
 int i64h_kattn(const i64h_kattn_args* d, void* stream);
+
+/* ---- attention with separate keys and values over one cached row per token --------------------------------------------------------------
+ * i64h_kv_prep, per row t of the projections P:  q = P[t, q_off : + heads * dim], k = P[t, k_off : + kv_heads * dim], v = P[t, v_off : + kv_heads * vdim];
+ *   cache row (slot, position) <- per key head g: [v_g (vdim) | k_g (dim)]   (cache == NULL: nothing is written - a layer that attends over
+ *   the rows another layer cached);   Q[t, h, :] = [0 (vdim) | q_h * scale (dim)].
+ * With these i64h_kattn (vdim > 0) computes softmax_j(Q . k_j + bias) v_j: the zeros make the value columns drop out of the score. */
+typedef struct {
+    const float* P;
+    int64_t ldp;
+    int32_t q_off, k_off, v_off;
+    int32_t heads, kv_heads, dim, vdim;
+    float scale;
+    const int32_t* positions;
+    const int32_t* slot_ids;
+    const int32_t* block_table;
+    int32_t max_blocks_per_seq, block_size;
+    void* cache;
+    int32_t cache_dtype;
+    float* Q;
+    int64_t n;
+} i64h_kv_prep_args;
+int i64h_kv_prep(const i64h_kv_prep_args* d, void* stream);
+
+/* ---- gated linear recurrence (linear attention with a decay per key channel) ----------------------------------------------------------------
+ * Per sequence and head a (dim x vdim) matrix S in fp32:   S <- diag(f_t) S + k_t v_t^T,   o_t = S^T q_t,
+ * q_t = P[t, q_off + a * dim : + dim], f_t likewise at f_off, v_t = P[t, v_off + a * vdim : + vdim];  k_t = P[...k_off...] or, with k_off < 0,
+ * k_t = 1 - f_t (the forget gate also decides what is written).  state fp32 [slots, heads, vdim, dim] (S transposed; dim <= 256).
+ * i64h_gla_gates prepares q and f in place:  q <- q_act ? silu(q) : q;   f <- lower + (1 - lower) * sigmoid(f)   (lower fp32 [heads * dim] or NULL = 0).
+ * All arithmetic fp32, the tokens of a sequence strictly in their order. */
+typedef struct {
+    float* P;
+    int64_t ldp;
+    int32_t q_off, f_off, k_off, v_off;
+    int32_t heads, dim, vdim;
+    const float* lower;
+    int32_t q_act;
+    const int32_t* seg_start;
+    int32_t nseg;
+    const int32_t* positions;
+    const int32_t* slot_ids;
+    float* state;
+    float* out;          /* fp32 [n, heads * vdim], row stride ldo */
+    int64_t ldo;
+    int64_t n;
+} i64h_gla_args;
+int i64h_gla_gates(const i64h_gla_args* d, void* stream);
+int i64h_gla_scan(const i64h_gla_args* d, void* stream);
+
+/* ---- router: softmax scores, corrected choice, groups of neighbours, top-k ---------------------------------------------------------------------
+ * Per row t of logits (fp32, row stride ld, E entries):  s = softmax(logits[t]);  choice = s + correction (correction may be NULL);
+ * with groups > 1 the E entries form `groups` equal groups of neighbours, a group's score is its largest choice and only the entries of
+ * the `keep` best groups can be chosen;  idx[t, :] = the `top` entries with the largest choice (ties: the lower index), in that order;
+ * wgt[t, k] = s[idx[t, k]] / (sum_k s[idx[t, k]] + 1e-20) * scale.   E <= 1024, top <= 32. */
+typedef struct {
+    const float* logits;
+    int64_t ld;
+    int32_t E;
+    const float* correction;
+    int32_t groups, keep, top;
+    float scale;
+    int32_t* idx;
+    float* wgt;
+    int64_t n;
+} i64h_route_args;
+int i64h_route_topk(const i64h_route_args* d, void* stream);
+
+/* ---- mixture of experts: rows per expert, and the weighted sum ----------------------------------------------------------------------------------
+ * i64h_moe_plan: from idx int32 [n, top] (entries >= experts are not experts and get no row) the (token, choice) pairs grouped by expert:
+ *   group_off int32 [experts + 1] (ascending offsets), pair_token int32 [n * top] (the token of every grouped row, the a_rows of a grouped
+ *   Linear), pair_row int32 [n, top] (where the pair's row lies, -1 for a non-expert).  The order of rows inside a group is not fixed;
+ *   no result depends on it.  One launch of one workgroup; experts <= 4096.
+ * i64h_moe_combine: out[t, :] = sum_k wgt[t, k] * (pair_row[t, k] >= 0 ? Y[pair_row[t, k], :] : h[t, :]) + (shared ? shared[t, :] : 0),
+ *   summed in the order k = 0 .. top - 1, the shared row last.  Y fp32 [pairs, W]. */
+typedef struct {
+    const int32_t* idx;
+    int64_t n;
+    int32_t top, experts;
+    int32_t* group_off;
+    int32_t* pair_token;
+    int32_t* pair_row;
+} i64h_moe_plan_args;
+int i64h_moe_plan(const i64h_moe_plan_args* d, void* stream);
+typedef struct {
+    const float* Y;
+    const int32_t* pair_row;
+    const float* wgt;
+    const float* h;
+    const float* shared;
+    float* out;
+    int64_t n;
+    int32_t top, W;
+} i64h_moe_combine_args;
+int i64h_moe_combine(const i64h_moe_combine_args* d, void* stream);
 
 /* ---- sampling --------------------------------------------------------------------------------------------------------------
  * out[r] = a token drawn from row r of logits fp32 [rows, V]: temperature[r] <= 0 -> the first index of the maximum (greedy);

@@ -223,6 +223,12 @@ DENSE_SIGNATURES: Dict[str, str] = {
     "i64h_mingru_scan": "pp",
     "i64h_kattn_prep": "pp",
     "i64h_kattn": "pp",
+    "i64h_kv_prep": "pp",
+    "i64h_gla_gates": "pp",
+    "i64h_gla_scan": "pp",
+    "i64h_route_topk": "pp",
+    "i64h_moe_plan": "pp",
+    "i64h_moe_combine": "pp",
 }
 
 
@@ -230,7 +236,7 @@ class Linear(ctypes.Structure):
     """Mirror of i64h_linear (include/i64h_dense.h)."""
     _fields_ = [("A", _P), ("lda", _L), ("a_rows", _P), ("W", _P), ("C", _P), ("ldc", _L), ("M", _L), ("N", _I), ("K", _I), ("batch", _I),
                 ("a_batch", _L), ("w_batch", _L), ("c_batch", _L), ("exact", _I), ("epilogue", _I), ("E", _P), ("lde", _L), ("e_batch", _L),
-                ("softcap", _F), ("bias", _P), ("bias_batch", _L), ("scale", _F)]
+                ("softcap", _F), ("bias", _P), ("bias_batch", _L), ("scale", _F), ("act_a", _F), ("act_b", _F), ("group_off", _P)]
 
 
 class PostNorm(ctypes.Structure):
@@ -258,7 +264,7 @@ class LatentAttn(ctypes.Structure):
 class EmbedBigram(ctypes.Structure):
     """Mirror of i64h_embed_bigram_args (include/i64h_dense.h)."""
     _fields_ = [("ids", _P), ("positions", _P), ("slot_ids", _P), ("table", _P), ("V", _L), ("W", _I), ("bigram", _P), ("buckets", _L),
-                ("mul_prev", _L), ("mul_cur", _L), ("prev_token", _P), ("out", _P), ("copies", _I), ("n", _L)]
+                ("mul_prev", _L), ("mul_cur", _L), ("prev_token", _P), ("out", _P), ("copies", _I), ("n", _L), ("pos_table", _P), ("pos_rows", _L)]
 
 
 class Streams(ctypes.Structure):
@@ -271,7 +277,7 @@ class Streams(ctypes.Structure):
 class CausalConv(ctypes.Structure):
     """Mirror of i64h_causal_conv_args (include/i64h_dense.h)."""
     _fields_ = [("P", _P), ("ldp", _L), ("off", _I), ("channels", _I), ("taps", _I), ("w", _P), ("bias", _P), ("positions", _P), ("slot_ids", _P),
-                ("state", _P), ("out", _P), ("ldo", _L), ("n", _L)]
+                ("state", _P), ("out", _P), ("ldo", _L), ("n", _L), ("mode", _I)]
 
 
 class SsmScan(ctypes.Structure):
@@ -303,7 +309,37 @@ class KAttn(ctypes.Structure):
     """Mirror of i64h_kattn_args (include/i64h_dense.h)."""
     _fields_ = [("Q", _P), ("cache", _P), ("cache_dtype", _I), ("kscale", _P), ("block_table", _P), ("max_blocks_per_seq", _I), ("block_size", _I),
                 ("slot_ids", _P), ("positions", _P), ("chunk", _I), ("bias", _P), ("bias_rows", _I), ("sink", _I), ("out", _P), ("n", _L), ("heads", _I),
-                ("kv_heads", _I), ("dim", _I), ("mode", _I), ("splits", _I), ("workspace", _P)]
+                ("kv_heads", _I), ("dim", _I), ("mode", _I), ("splits", _I), ("workspace", _P), ("vdim", _I)]
+
+
+class KvPrep(ctypes.Structure):
+    """Mirror of i64h_kv_prep_args (include/i64h_dense.h)."""
+    _fields_ = [("P", _P), ("ldp", _L), ("q_off", _I), ("k_off", _I), ("v_off", _I), ("heads", _I), ("kv_heads", _I), ("dim", _I), ("vdim", _I),
+                ("scale", _F), ("positions", _P), ("slot_ids", _P), ("block_table", _P), ("max_blocks_per_seq", _I), ("block_size", _I),
+                ("cache", _P), ("cache_dtype", _I), ("Q", _P), ("n", _L)]
+
+
+class Gla(ctypes.Structure):
+    """Mirror of i64h_gla_args (include/i64h_dense.h)."""
+    _fields_ = [("P", _P), ("ldp", _L), ("q_off", _I), ("f_off", _I), ("k_off", _I), ("v_off", _I), ("heads", _I), ("dim", _I), ("vdim", _I),
+                ("lower", _P), ("q_act", _I), ("seg_start", _P), ("nseg", _I), ("positions", _P), ("slot_ids", _P), ("state", _P), ("out", _P),
+                ("ldo", _L), ("n", _L)]
+
+
+class Route(ctypes.Structure):
+    """Mirror of i64h_route_args (include/i64h_dense.h)."""
+    _fields_ = [("logits", _P), ("ld", _L), ("E", _I), ("correction", _P), ("groups", _I), ("keep", _I), ("top", _I), ("scale", _F), ("idx", _P),
+                ("wgt", _P), ("n", _L)]
+
+
+class MoePlan(ctypes.Structure):
+    """Mirror of i64h_moe_plan_args (include/i64h_dense.h)."""
+    _fields_ = [("idx", _P), ("n", _L), ("top", _I), ("experts", _I), ("group_off", _P), ("pair_token", _P), ("pair_row", _P)]
+
+
+class MoeCombine(ctypes.Structure):
+    """Mirror of i64h_moe_combine_args (include/i64h_dense.h)."""
+    _fields_ = [("Y", _P), ("pair_row", _P), ("wgt", _P), ("h", _P), ("shared", _P), ("out", _P), ("n", _L), ("top", _I), ("W", _I)]
 
 
 _dense: Optional[ctypes.CDLL] = None

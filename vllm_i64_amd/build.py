@@ -2,7 +2,8 @@
 
 libi64hip.so        the quantized token-routed-MoE forward (include/i64h.h)
 libi64hip_dense.so  models with bf16 weights and a 32-bit residual: Linear, gated post-norm, latent attention, multi-stream
-                    residual, state-space / gated recurrences, key-valued chunked attention, sampling
+                    residual, state-space / gated recurrences, key-valued chunked attention, attention with separate keys and values,
+                    gated linear recurrence, expert routing and grouped expert Linears, sampling
                     (include/i64h_dense.h) - a library of its own, so that serving such a model builds nothing else
 """
 from __future__ import annotations
@@ -16,7 +17,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libi64hip.so")
 DENSE_OUT = os.path.join(HERE, "libi64hip_dense.so")
-DENSE_SOURCES = ["i64h_api.hip", "i64h_dense.hip", "i64h_latent.hip", "i64h_hybrid.hip"]
+DENSE_SOURCES = ["i64h_api.hip", "i64h_dense.hip", "i64h_latent.hip", "i64h_hybrid.hip", "i64h_blocks.hip"]
 SOURCES = ["i64h_api.hip", "i64h_route.hip", "i64h_quant.hip", "i64h_norm.hip", "i64h_gemm.hip", "i64h_gemm_os.hip", "i64h_attn.hip", "i64h_moe.hip", "i64h_fp8.hip", "i64h_kv.hip", "i64h_decode.hip", "i64h_variants.hip", "i64h_group_f32.hip", "i64h_lmhead.hip"]
 # -ffp-contract=off: a*b+c stays two roundings unless the source says fmaf, so fp32 element-wise math has the
 # same rounding steps as the reference's CPU ops.

@@ -116,12 +116,58 @@ class LatentAttentionConfig:
 @dataclass
 class DenseMlpConfig:
     ff: int
+    kind: str = "dense"
 
     @classmethod
     def from_dict(cls, m: dict) -> "DenseMlpConfig":
         if m.get("kind", "dense") != "dense":
             raise ValueError(f"feed-forward kind '{m.get('kind')}' is not built")
         return cls(ff=int(m["ff"]))
+
+    def to_dict(self) -> dict:
+        return {"kind": "dense", "ff": self.ff}
+
+
+@dataclass
+class MoeMlpConfig:
+    """Mixture of gated feed-forward experts.  The router scores `experts + identity` entries (the last `identity` of them hand their
+    input through and have no tensors); its entries form `groups` equal groups of neighbours of which the `keep` best (by their largest
+    corrected score) may be chosen from; every token takes `top` entries, weighted by their uncorrected scores, renormalised and
+    multiplied by `scale`.  shared_ff > 0: one more expert of that size runs for every token."""
+    ff: int
+    experts: int
+    top: int
+    identity: int = 0
+    groups: int = 1
+    keep: int = 1
+    scale: float = 1.0
+    shared_ff: int = 0
+    kind: str = "moe"
+
+    @property
+    def entries(self) -> int:
+        return self.experts + self.identity
+
+    @classmethod
+    def from_dict(cls, m: dict) -> "MoeMlpConfig":
+        r = m["router"]
+        g = r.get("groups") or {}
+        c = cls(ff=int(m["expert"]["ff"]), experts=int(r["experts"]), top=int(r["top"]), identity=int(r.get("identity", 0)), groups=int(g.get("count", 1)),
+                keep=int(g.get("keep", g.get("count", 1))), scale=float(r.get("scale", 1.0)), shared_ff=int((m.get("shared") or {}).get("ff", 0)))
+        if min(c.ff, c.experts, c.top, c.groups, c.keep) <= 0 or c.identity < 0 or c.shared_ff < 0 or c.top > c.entries or c.entries % c.groups or \
+                c.keep > c.groups or c.keep * (c.entries // c.groups) < c.top:
+            raise ValueError(f"mixture of experts: bad sizes {m}")
+        return c
+
+    def to_dict(self) -> dict:
+        d = {"kind": "moe", "expert": {"ff": self.ff},
+             "router": {"experts": self.experts, "top": self.top, "identity": self.identity, "scale": self.scale, "groups": {"count": self.groups, "keep": self.keep}}}
+        if self.shared_ff:
+            d["shared"] = {"ff": self.shared_ff}
+        return d
+
+
+MLPS = {"dense": DenseMlpConfig, "moe": MoeMlpConfig}
 
 
 @dataclass
@@ -217,7 +263,56 @@ class ParallelMixerConfig:
         return {"left": self.left.to_dict(), "right": self.right.to_dict()}
 
 
-MIXERS = {"latent_attention": LatentAttentionConfig, "mamba2": Mamba2Config, "parallel": ParallelMixerConfig}
+@dataclass
+class Hgrn2Config:
+    """Gated linear recurrence: per head a (dim x vdim) matrix with a forget gate per key channel, bounded below by a learned value; what
+    the gate does not keep is written (the key is one minus the gate).  The head outputs pass an RMS norm over vdim."""
+    heads: int
+    dim: int
+    vdim: int
+
+    @classmethod
+    def from_dict(cls, m: dict) -> "Hgrn2Config":
+        c = cls(heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])))
+        if min(c.heads, c.dim, c.vdim) <= 0:
+            raise ValueError(f"hgrn2: bad sizes {m}")
+        return c
+
+    def to_dict(self) -> dict:
+        return {"heads": self.heads, "dim": self.dim, "vdim": self.vdim}
+
+
+@dataclass
+class BiasedAttentionConfig:
+    """Causal attention with grouped key / value heads, separate key and value sizes, no rotation, and a learned bias by bucketed distance
+    (as many buckets as the table has rows, logarithmic up to bias_max).  kv_from: the layer whose cached keys and values this layer
+    attends over instead of projecting its own."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    bias_max: float = 0.0
+    kv_from: "int | None" = None
+
+    @classmethod
+    def from_dict(cls, m: dict) -> "BiasedAttentionConfig":
+        src = m.get("kv_from")
+        c = cls(heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])), dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])),
+                scale=float(m["scale"]), bias_max=float(m.get("bias_max", 0.0)), kv_from=int(src) if src is not None else None)
+        if min(c.heads, c.kv_heads, c.dim, c.vdim) <= 0 or c.heads % c.kv_heads:
+            raise ValueError(f"attention: bad sizes {m}")
+        return c
+
+    def to_dict(self) -> dict:
+        d = {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim, "scale": self.scale, "bias_max": self.bias_max}
+        if self.kv_from is not None:
+            d["kv_from"] = self.kv_from
+        return d
+
+
+MIXERS = {"latent_attention": LatentAttentionConfig, "mamba2": Mamba2Config, "parallel": ParallelMixerConfig, "hgrn2": Hgrn2Config,
+          "attention": BiasedAttentionConfig}
 
 
 @dataclass
@@ -234,7 +329,9 @@ class DecoderLayerConfig:
             raise ValueError(f"layer type '{kind}' is not built (known: {sorted(MIXERS)})")
         mlp = d.get("mlp")
         share = d.get("weights_of")
-        return cls(type=kind, mixer=MIXERS[kind].from_dict(d["mixer"]), mlp=DenseMlpConfig.from_dict(mlp) if mlp else None,
+        if mlp and mlp.get("kind", "dense") not in MLPS:
+            raise ValueError(f"feed-forward kind '{mlp.get('kind')}' is not built (known: {sorted(MLPS)})")
+        return cls(type=kind, mixer=MIXERS[kind].from_dict(d["mixer"]), mlp=MLPS[mlp.get("kind", "dense")].from_dict(mlp) if mlp else None,
                    weights_of=int(share) if share is not None else None)
 
 
@@ -358,3 +455,61 @@ class DogalornConfig:
         if self.bigram is not None:
             d["embedding"] = {"bigram": {"buckets": self.bigram.buckets, "mul_prev": self.bigram.mul_prev, "mul_cur": self.bigram.mul_cur}}
         return d
+
+
+# ---------------------------------------------------------------------------------------------------------------------------
+# Zabutar: sandwich-norm decoder (an RMS norm in front of and behind every sublayer, weights stored as distances from one) with
+# learned absolute positions, a short causal convolution added to every sublayer's input, and layers that mix either by a gated
+# linear recurrence or by attention with a distance bias (some attending over another layer's cached keys and values); dense
+# feed-forwards with a two-branch quadratic / exponential activation, or mixtures of gated experts.  Every size and constant comes
+# from the checkpoint's config.json.
+# ---------------------------------------------------------------------------------------------------------------------------
+@dataclass
+class ZabutarConfig:
+    vocab: int
+    width: int
+    layers: list
+    max_positions: int
+    norm_eps: float = 1e-6
+    canon_taps: int = 1
+    name: str = "Zabutar"
+
+    LAYER_TYPES = ("hgrn2", "attention")
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def vocab_size(self) -> int:
+        return self.vocab
+
+    @property
+    def max_pos(self) -> int:
+        """Positions are rows of a learned table: a sequence ends where the table does."""
+        return self.max_positions
+
+    @classmethod
+    def from_dict(cls, d: dict) -> "ZabutarConfig":
+        layers = [DecoderLayerConfig.from_dict(l) for l in d["layers"]]
+        c = cls(vocab=int(d["vocab"]), width=int(d["width"]), layers=layers, max_positions=int(d["max_positions"]),
+                norm_eps=float((d.get("norm") or {}).get("eps", 1e-6)), canon_taps=int((d.get("canon") or {}).get("taps", 1)),
+                name=str(d.get("architecture", "Zabutar")))
+        if min(c.vocab, c.width, c.max_positions, c.canon_taps) <= 0:
+            raise ValueError("bad sizes")
+        for i, l in enumerate(layers):
+            if l.type not in cls.LAYER_TYPES:
+                raise ValueError(f"layer {i}: type '{l.type}' is not part of this design (known: {cls.LAYER_TYPES})")
+            if l.weights_of is not None:
+                raise ValueError(f"layer {i}: this design has no layers that borrow tensors")
+            if l.type == "attention" and l.mixer.kv_from is not None:
+                j, m = l.mixer.kv_from, l.mixer
+                o = layers[j].mixer if 0 <= j < i and layers[j].type == "attention" else None
+                if o is None or o.kv_from is not None or (o.kv_heads, o.dim, o.vdim) != (m.kv_heads, m.dim, m.vdim):
+                    raise ValueError(f"layer {i}: takes keys and values from layer {j}, which is no earlier attention layer with projections of its own and the same sizes")
+        return c
+
+    def to_dict(self) -> dict:
+        return {"architecture": "Zabutar", "vocab": self.vocab, "width": self.width, "max_positions": self.max_positions, "norm": {"eps": self.norm_eps},
+                "canon": {"taps": self.canon_taps},
+                "layers": [{"type": l.type, "mixer": l.mixer.to_dict(), "mlp": l.mlp.to_dict() if l.mlp else None} for l in self.layers]}

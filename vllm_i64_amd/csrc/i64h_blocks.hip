@@ -1,0 +1,343 @@
+// Kernels of libi64hip_dense.so for gated linear recurrences and mixtures of experts (include/i64h_dense.h):
+//   gla_gates_kernel   : query activation and bounded forget gate, in place on the projection rows
+//   gla_scan_kernel    : linear attention with a decay per key channel, a head's matrix in registers (16 lanes per value column)
+//   route_topk_kernel  : softmax scores, corrected choice, groups of neighbours, top-k and normalised weights, one wave per row
+//   moe_plan_kernel    : (token, choice) pairs grouped by expert: offsets, the token of every grouped row, the row of every pair
+//   moe_combine_kernel : weighted sum of the chosen experts' rows, pass-through entries and the shared expert's row
+// A row continues the row before it iff slot and position say so; state is taken as empty at position 0.  All arithmetic fp32.
+#include "i64h_common.h"
+#include "i64h_dense.h"
+
+__device__ __forceinline__ float bl_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+// ---------------------------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void gla_gates_kernel(const i64h_gla_args p) {
+    const int64_t t = blockIdx.y;
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= p.heads * p.dim) return;
+    float* row = p.P + t * p.ldp;
+    if (p.q_act) {
+        const float q = row[p.q_off + c];
+        row[p.q_off + c] = q * bl_sigmoid(q);
+    }
+    const float lo = p.lower ? p.lower[c] : 0.0f;
+    row[p.f_off + c] = lo + (1.0f - lo) * bl_sigmoid(row[p.f_off + c]);
+}
+
+// One workgroup per (head, 16 * CPT value columns, run of rows).  The 16 lanes of a DPP row share CPT neighbouring value columns and hold
+// KPT consecutive key channels of each in registers; a wave has four such rows.  Per token a lane loads its slices of the query, the
+// decay and (where it is not one minus the decay) the key once for its CPT columns - the next token's while this one is computed -,
+// updates its states with fused multiply-adds and the row sums the partial outputs with DPP moves: no LDS and no barrier, the tokens of
+// a run strictly in their order (the same sums in the same order however a prompt is cut).  State layout [slot, head, value column,
+// key channel].
+template <int KPT, int CPT>
+__global__ __launch_bounds__(256) void gla_scan_kernel(const i64h_gla_args p, const int ctiles, const int vec) {
+    const int N = p.dim, P = p.vdim;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int nlane = lane & 15, cl = lane >> 4;
+    const int a = blockIdx.x / ctiles, seg = blockIdx.y;
+    const int cbase = (blockIdx.x % ctiles) * 16 * CPT + (w * 4 + cl) * CPT;
+    const int64_t r0 = p.seg_start[seg], r1 = p.seg_start[seg + 1];
+    if (r1 <= r0) return;
+    const int n0 = nlane * KPT;
+    float S[CPT][KPT];
+    float* gS = p.state + ((int64_t)p.slot_ids[r0] * p.heads + a) * P * N + n0;      // + column * N
+    const bool fresh = p.positions[r0] == 0;
+#pragma unroll
+    for (int j = 0; j < CPT; ++j) {
+        const bool cok = cbase + j < P;
+        const float* src = gS + (int64_t)(cok ? cbase + j : 0) * N;
+#pragma unroll
+        for (int k = 0; k < KPT; ++k) S[j][k] = (!fresh && cok && n0 + k < N) ? src[k] : 0.0f;
+    }
+    const int qoff = p.q_off + a * N + n0, foff = p.f_off + a * N + n0, koff = p.k_off >= 0 ? p.k_off + a * N + n0 : -1;
+    struct Tok {
+        float q[KPT], f[KPT], k[KPT], v[CPT];
+    };
+    auto fetch = [&](int64_t t, Tok& u) {
+        const float* row = p.P + t * p.ldp;
+        if (vec) {      // KPT % 4 == 0 and every slice starts at a multiple of four floats and lies inside the row
+#pragma unroll
+            for (int k = 0; k < KPT; k += 4) {
+                float4 q = make_float4(0, 0, 0, 0), f = make_float4(1, 1, 1, 1), kk = q;
+                if (n0 + k < N) {
+                    q = *(const float4*)(row + qoff + k);
+                    f = *(const float4*)(row + foff + k);
+                    if (koff >= 0) kk = *(const float4*)(row + koff + k);
+                }
+                u.q[k] = q.x, u.q[k + 1] = q.y, u.q[k + 2] = q.z, u.q[k + 3] = q.w;
+                u.f[k] = f.x, u.f[k + 1] = f.y, u.f[k + 2] = f.z, u.f[k + 3] = f.w;
+                u.k[k] = kk.x, u.k[k + 1] = kk.y, u.k[k + 2] = kk.z, u.k[k + 3] = kk.w;
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < KPT; ++k) {
+                const bool ok = n0 + k < N;
+                u.q[k] = ok ? row[qoff + k] : 0.0f;
+                u.f[k] = ok ? row[foff + k] : 1.0f;
+                u.k[k] = (ok && koff >= 0) ? row[koff + k] : 0.0f;
+            }
+        }
+        if (koff < 0) {
+#pragma unroll
+            for (int k = 0; k < KPT; ++k) u.k[k] = 1.0f - u.f[k];
+        }
+#pragma unroll
+        for (int j = 0; j < CPT; ++j) u.v[j] = cbase + j < P ? row[p.v_off + a * P + cbase + j] : 0.0f;
+    };
+    auto step = [&](int64_t t, const Tok& u) {
+#pragma unroll
+        for (int j = 0; j < CPT; ++j) {
+            float part = 0.0f;
+#pragma unroll
+            for (int k = 0; k < KPT; ++k) {
+                S[j][k] = fmaf(u.f[k], S[j][k], u.k[k] * u.v[j]);
+                part = fmaf(S[j][k], u.q[k], part);
+            }
+            part = group_sum(part, 16);
+            if (nlane == 0 && cbase + j < P) p.out[t * p.ldo + a * P + cbase + j] = part;
+        }
+    };
+    Tok u0, u1;
+    fetch(r0, u0);
+    for (int64_t t = r0; t < r1; t += 2) {
+        if (t + 1 < r1) fetch(t + 1, u1);
+        step(t, u0);
+        if (t + 1 < r1) {
+            if (t + 2 < r1) fetch(t + 2, u0);
+            step(t + 1, u1);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < CPT; ++j) {
+        if (cbase + j >= P) continue;
+        float* dst = gS + (int64_t)(cbase + j) * N;
+#pragma unroll
+        for (int k = 0; k < KPT; ++k)
+            if (n0 + k < N) dst[k] = S[j][k];
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------------------
+// the lane that holds the largest value, ties to the lower index; (value, index) pairs with index < 0 do not take part
+__device__ __forceinline__ int bl_wave_argmax(float v, int idx, float& best) {
+    best = wave_max(idx >= 0 ? v : -INFINITY);
+    const int cand = (idx >= 0 && v == best) ? idx : 0x7fffffff;
+    return -wave_max_i(-cand);
+}
+
+#define RT_MAX_TOP 32
+__global__ __launch_bounds__(256) void route_topk_kernel(const i64h_route_args p) {
+    extern __shared__ float rt_lds[];   // per wave: [E] scores, [E] choice values, [groups] group flags
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+    const int64_t t = (int64_t)blockIdx.x * 4 + wid;
+    if (t >= p.n) return;     // (a whole wave leaves; no workgroup barrier below)
+    const int E = p.E, G = p.groups > 1 ? p.groups : 1, gsz = E / G;
+    // volatile: lanes read what another lane of the wave wrote (one wave: program order is enough, no barrier)
+    volatile float* sc = rt_lds + (size_t)wid * (2 * E + G);
+    volatile float* ch = sc + E;
+    volatile float* gflag = ch + E;
+    const float* z = p.logits + t * p.ld;
+    float mx = -INFINITY;
+    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
+    mx = wave_max(mx);
+    float sum = 0.0f;
+    for (int e = lane; e < E; e += 64) {
+        const float v = expf(z[e] - mx);
+        sc[e] = v;
+        sum += v;
+    }
+    sum = wave_sum(sum);
+    for (int e = lane; e < E; e += 64) {
+        const float s = sc[e] / sum;
+        sc[e] = s;
+        ch[e] = p.correction ? s + p.correction[e] : s;
+    }
+    if (G > 1) {   // a group's score: its largest choice value; the `keep` best groups stay, the entries of the others cannot be chosen
+        for (int g = lane; g < G; g += 64) {
+            float b = -INFINITY;
+            for (int i = 0; i < gsz; ++i) b = fmaxf(b, ch[g * gsz + i]);
+            gflag[g] = b;
+        }
+        // (LDS traffic of one wave needs program order only)
+        for (int r = 0; r < p.keep; ++r) {
+            float bv = -INFINITY;
+            int bi = -1;
+            for (int g = lane; g < G; g += 64) {
+                const float v = gflag[g];
+                if (!(v != v) && v != INFINITY && (bi < 0 || v > bv)) bv = v, bi = g;     // +inf marks a group already kept
+            }
+            float best;
+            const int pick = bl_wave_argmax(bv, bi, best);
+            if (pick != 0x7fffffff && lane == 0) gflag[pick] = INFINITY;
+        }
+        for (int e = lane; e < E; e += 64)
+            if (gflag[e / gsz] != INFINITY) ch[e] = -INFINITY;
+    }
+    float wsum = 0.0f;
+    float mine_w = 0.0f;      // lane k keeps the k-th choice
+    int mine_i = 0;
+    for (int k = 0; k < p.top; ++k) {
+        float bv = -INFINITY;
+        int bi = -1;
+        for (int e = lane; e < E; e += 64) {
+            const float v = ch[e];
+            if (v == v && (bi < 0 || v > bv)) bv = v, bi = e;
+        }
+        float best;
+        int pick = bl_wave_argmax(bv, bi, best);
+        if (pick == 0x7fffffff) pick = 0;
+        const float s = sc[pick];
+        wsum += s;
+        if (lane == k) mine_w = s, mine_i = pick;
+        if (lane == 0) ch[pick] = __builtin_nanf("");     // taken: out of every later comparison
+    }
+    if (lane < p.top) {
+        p.idx[t * p.top + lane] = mine_i;
+        p.wgt[t * p.top + lane] = mine_w / (wsum + 1e-20f) * p.scale;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(1024) void moe_plan_kernel(const i64h_moe_plan_args p) {
+    extern __shared__ int pl_lds[];   // [experts + 1] counts, then offsets; [experts] cursors
+    int* cnt = pl_lds;
+    int* cur = pl_lds + p.experts + 1;
+    const int tid = threadIdx.x;
+    const int64_t pairs = p.n * p.top;
+    for (int e = tid; e <= p.experts; e += 1024) cnt[e] = 0;
+    __syncthreads();
+    for (int64_t i = tid; i < pairs; i += 1024) {
+        const int e = p.idx[i];
+        if (e >= 0 && e < p.experts) atomicAdd(&cnt[e], 1);
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int run = 0;
+        for (int e = 0; e < p.experts; ++e) {
+            const int c = cnt[e];
+            cnt[e] = run;
+            cur[e] = run;
+            run += c;
+        }
+        cnt[p.experts] = run;
+    }
+    __syncthreads();
+    for (int e = tid; e <= p.experts; e += 1024) p.group_off[e] = cnt[e];
+    for (int64_t i = tid; i < pairs; i += 1024) {
+        const int e = p.idx[i];
+        int r = -1;
+        if (e >= 0 && e < p.experts) {
+            r = atomicAdd(&cur[e], 1);
+            p.pair_token[r] = (int)(i / p.top);
+        }
+        p.pair_row[i] = r;
+    }
+}
+
+__global__ __launch_bounds__(256) void moe_combine_kernel(const i64h_moe_combine_args p) {
+    const int64_t t = blockIdx.x;
+    const int W = p.W;
+    for (int c = threadIdx.x; c < W; c += 256) {
+        float a = 0.0f;
+        for (int k = 0; k < p.top; ++k) {
+            const int r = p.pair_row[t * p.top + k];
+            const float v = r >= 0 ? p.Y[(int64_t)r * W + c] : p.h[t * W + c];
+            a += p.wgt[t * p.top + k] * v;
+        }
+        if (p.shared) a += p.shared[t * W + c];
+        p.out[t * W + c] = a;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------------------
+extern "C" {
+
+static int gla_check(const i64h_gla_args& d, const char* what) {
+    I64H_CHECK_ARG(d.heads > 0 && d.dim > 0 && d.vdim > 0 && d.n >= 0, "%s: heads %d, dim %d, vdim %d", what, d.heads, d.dim, d.vdim);
+    I64H_CHECK_ARG(d.P && d.q_off >= 0 && d.f_off >= 0 && d.v_off >= 0, "%s: null operand or negative column", what);
+    return 0;
+}
+
+int i64h_gla_gates(const i64h_gla_args* dp, void* stream) {
+    I64H_CHECK_ARG(dp != nullptr, "gla_gates: no descriptor");
+    const i64h_gla_args& d = *dp;
+    if (gla_check(d, "gla_gates")) return 1;
+    I64H_CHECK_ARG(d.n <= 65535, "gla_gates: %lld rows in one launch (at most 65535)", (long long)d.n);
+    if (d.n == 0) return 0;
+    hipLaunchKernelGGL(gla_gates_kernel, dim3((unsigned)((d.heads * d.dim + 255) / 256), (unsigned)d.n), dim3(256), 0, (hipStream_t)stream, d);
+    I64H_CHECK_LAUNCH();
+    return 0;
+}
+
+int i64h_gla_scan(const i64h_gla_args* dp, void* stream) {
+    I64H_CHECK_ARG(dp != nullptr, "gla_scan: no descriptor");
+    const i64h_gla_args& d = *dp;
+    if (gla_check(d, "gla_scan")) return 1;
+    I64H_CHECK_ARG(d.seg_start && d.positions && d.slot_ids && d.state && d.out, "gla_scan: null operand");
+    I64H_CHECK_ARG(d.dim <= 16 * 16, "gla_scan: dim %d above 256", d.dim);
+    I64H_CHECK_ARG(d.nseg <= 65535, "gla_scan: %d runs in one launch", d.nseg);
+    if (d.nseg <= 0 || d.n == 0) return 0;
+    const int kpt = (d.dim + 15) / 16;
+    const int cpt = d.vdim > 16 ? 2 : 1;             // columns per lane: query, decay and key are loaded once for both
+    const int ctiles = (d.vdim + 16 * cpt - 1) / (16 * cpt);
+    const dim3 grid((unsigned)(d.heads * ctiles), (unsigned)d.nseg);
+    auto launch = [&](auto kern, int K) {
+        const int vec = K % 4 == 0 && d.dim % 4 == 0 && d.ldp % 4 == 0 && d.q_off % 4 == 0 && d.f_off % 4 == 0 && (d.k_off < 0 || d.k_off % 4 == 0) &&
+                        (uintptr_t)d.P % 16 == 0;
+        hipLaunchKernelGGL(kern, grid, dim3(256), 0, (hipStream_t)stream, d, ctiles, vec);
+    };
+    if (cpt == 2) {
+        if (kpt <= 1) launch(gla_scan_kernel<1, 2>, 1);
+        else if (kpt <= 2) launch(gla_scan_kernel<2, 2>, 2);
+        else if (kpt <= 4) launch(gla_scan_kernel<4, 2>, 4);
+        else if (kpt <= 8) launch(gla_scan_kernel<8, 2>, 8);
+        else launch(gla_scan_kernel<16, 2>, 16);
+    } else {
+        if (kpt <= 1) launch(gla_scan_kernel<1, 1>, 1);
+        else if (kpt <= 2) launch(gla_scan_kernel<2, 1>, 2);
+        else if (kpt <= 4) launch(gla_scan_kernel<4, 1>, 4);
+        else if (kpt <= 8) launch(gla_scan_kernel<8, 1>, 8);
+        else launch(gla_scan_kernel<16, 1>, 16);
+    }
+    I64H_CHECK_LAUNCH();
+    return 0;
+}
+
+int i64h_route_topk(const i64h_route_args* dp, void* stream) {
+    I64H_CHECK_ARG(dp != nullptr, "route_topk: no descriptor");
+    const i64h_route_args& d = *dp;
+    I64H_CHECK_ARG(d.E > 0 && d.E <= 1024 && d.top > 0 && d.top <= RT_MAX_TOP && d.top <= d.E, "route_topk: %d entries (at most 1024), top %d (at most %d)", d.E, d.top, RT_MAX_TOP);
+    I64H_CHECK_ARG(d.groups <= 1 || (d.E % d.groups == 0 && d.keep >= 1 && d.keep <= d.groups), "route_topk: %d entries in %d groups, %d kept", d.E, d.groups, d.keep);
+    I64H_CHECK_ARG(d.groups <= 1 || d.keep * (d.E / d.groups) >= d.top, "route_topk: %d kept groups of %d entries hold fewer than top %d", d.keep, d.E / (d.groups > 0 ? d.groups : 1), d.top);
+    I64H_CHECK_ARG(d.logits && d.idx && d.wgt && d.ld >= d.E, "route_topk: null operand or row stride below the entries");
+    if (d.n == 0) return 0;
+    const size_t lds = 4 * (size_t)(2 * d.E + (d.groups > 1 ? d.groups : 1)) * 4;
+    hipLaunchKernelGGL(route_topk_kernel, dim3((unsigned)((d.n + 3) / 4)), dim3(256), lds, (hipStream_t)stream, d);
+    I64H_CHECK_LAUNCH();
+    return 0;
+}
+
+int i64h_moe_plan(const i64h_moe_plan_args* dp, void* stream) {
+    I64H_CHECK_ARG(dp != nullptr, "moe_plan: no descriptor");
+    const i64h_moe_plan_args& d = *dp;
+    I64H_CHECK_ARG(d.experts > 0 && d.experts <= 4096 && d.top > 0 && d.n >= 0, "moe_plan: %d experts (at most 4096), top %d", d.experts, d.top);
+    I64H_CHECK_ARG(d.idx && d.group_off && d.pair_token && d.pair_row, "moe_plan: null operand");
+    I64H_CHECK_ARG(d.n * d.top < (1ll << 31), "moe_plan: too many pairs");
+    hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(1024), (size_t)(2 * d.experts + 1) * 4, (hipStream_t)stream, d);
+    I64H_CHECK_LAUNCH();
+    return 0;
+}
+
+int i64h_moe_combine(const i64h_moe_combine_args* dp, void* stream) {
+    I64H_CHECK_ARG(dp != nullptr, "moe_combine: no descriptor");
+    const i64h_moe_combine_args& d = *dp;
+    I64H_CHECK_ARG(d.top > 0 && d.W > 0 && d.n >= 0, "moe_combine: top %d, width %d", d.top, d.W);
+    I64H_CHECK_ARG(d.Y && d.pair_row && d.wgt && d.h && d.out, "moe_combine: null operand");
+    if (d.n == 0) return 0;
+    hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)d.n), dim3(256), 0, (hipStream_t)stream, d);
+    I64H_CHECK_LAUNCH();
+    return 0;
+}
+
+}  // extern "C"

@@ -31,10 +31,17 @@ __device__ __forceinline__ float dn_gelu_tanh(float z) {
 
 __device__ __forceinline__ float dn_gelu_erf(float z) { return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f)); }
 
+__device__ __forceinline__ float dn_xielu(float z, float a, float b) {
+    return z > 0.0f ? a * z * z + 0.5f * z : b * (expm1f(z) - z) + 0.5f * z;
+}
+constexpr bool dn_dual(int epi) { return epi == I64H_EPI_GELU_MUL || epi == I64H_EPI_SILU_MUL; }  // two accumulators: gate rows and up rows
+
 template <int EPI>
 __device__ __forceinline__ float dn_epilogue(const i64h_linear& p, float acc, float acc2, int64_t b, int64_t r, int c) {
     if (EPI == I64H_EPI_GELU_MUL) return dn_gelu_tanh(acc) * acc2;
+    if (EPI == I64H_EPI_SILU_MUL) return acc * dn_sigmoid(acc) * acc2;
     if (p.bias) acc += p.bias[b * p.bias_batch + c];
+    if (EPI == I64H_EPI_XIELU) return dn_xielu(acc, p.act_a, p.act_b);
     if (EPI == I64H_EPI_GELU_ERF) return dn_gelu_erf(acc);
     if (EPI == I64H_EPI_SCALE) return acc * p.scale;
     if (EPI == I64H_EPI_MUL_SIGMOID) return acc * dn_sigmoid(p.E[b * p.e_batch + r * p.lde + c]);
@@ -45,7 +52,7 @@ __device__ __forceinline__ float dn_epilogue(const i64h_linear& p, float acc, fl
 // ---------------------------------------------------------------------------------------------------------------------------
 template <bool EXACT, int EPI>
 __global__ __launch_bounds__(256) void linear_tile_kernel(const i64h_linear p, const int vecA, const int vecW) {
-    constexpr bool DUAL = EPI == I64H_EPI_GELU_MUL;
+    constexpr bool DUAL = dn_dual(EPI);
     constexpr int LD = EXACT ? 33 : 40;  // 33 words: conflict-free column reads; 40 halves = 80 bytes: 16-byte aligned fragments
     using T = typename std::conditional<EXACT, float, uint16_t>::type;
     __shared__ __attribute__((aligned(16))) T sA[2][64][LD];
@@ -54,9 +61,17 @@ __global__ __launch_bounds__(256) void linear_tile_kernel(const i64h_linear p, c
     const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
     const int wm = wid >> 1, wn = wid & 1;
     const int64_t b = blockIdx.z;
-    const int64_t m0 = (int64_t)blockIdx.y * 64;
+    int64_t m0 = (int64_t)blockIdx.y * 64;
     const int n0 = blockIdx.x * 64;
-    const int M = (int)min((int64_t)64, p.M - m0);  // rows of this tile
+    int64_t rows = p.M;
+    if (p.group_off) {   // this batch's share of the rows; m0 becomes the tile's first row among all rows
+        const int64_t g0 = p.group_off[b];
+        rows = min(rows, (int64_t)p.group_off[b + 1] - g0);
+        if (m0 >= rows) return;
+        rows += g0;
+        m0 += g0;
+    }
+    const int M = (int)min((int64_t)64, rows - m0);  // rows of this tile
     const int N = p.N, K = p.K;
     const int lr = tid >> 2, lc = (tid & 3) * 8;
     const bool aok = lr < M, bok = n0 + lr < N;
@@ -180,7 +195,7 @@ __global__ __launch_bounds__(256) void linear_tile_kernel(const i64h_linear p, c
 // 32-wide k step against 8 fragment reads - four times the 64 x 64 kernel's ratio), the same staging scheme.
 template <int EPI>
 __global__ __launch_bounds__(256) void linear_tile128_kernel(const i64h_linear p, const int vecA, const int vecW) {
-    constexpr bool DUAL = EPI == I64H_EPI_GELU_MUL;
+    constexpr bool DUAL = dn_dual(EPI);
     constexpr int LD = 40;
     __shared__ __attribute__((aligned(16))) uint16_t sA[2][128][LD];
     __shared__ __attribute__((aligned(16))) uint16_t sB[2][128][LD];
@@ -300,7 +315,7 @@ __global__ __launch_bounds__(256) void linear_tile128_kernel(const i64h_linear p
 // time, every lane 8 consecutive k of each per iteration (one 16-byte load per weight row), products in fp32.
 template <int EPI>
 __global__ __launch_bounds__(256) void linear_skinny_kernel(const i64h_linear p, const int cols_per_block) {
-    constexpr bool DUAL = EPI == I64H_EPI_GELU_MUL;
+    constexpr bool DUAL = dn_dual(EPI);
     constexpr int CPW = 4, MR = I64H_SKINNY_ROWS;
     extern __shared__ __attribute__((aligned(16))) uint16_t sa[];  // [M][K]
     const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
@@ -384,7 +399,7 @@ __global__ __launch_bounds__(256) void linear_skinny_kernel(const i64h_linear p,
 // Many small workgroups fill the chip where a launch has few 64-column tiles, and the weights stream exactly once.
 template <int EPI, int NW>
 __global__ __launch_bounds__(64 * NW) void linear_rows64_kernel(const i64h_linear p) {
-    constexpr bool DUAL = EPI == I64H_EPI_GELU_MUL;
+    constexpr bool DUAL = dn_dual(EPI);
     __shared__ float red[DUAL ? 2 : 1][NW][64][17];
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int n = lane & 15, kg = lane >> 4;
@@ -662,9 +677,11 @@ template <bool EXACT>
 static void launch_tile(const i64h_linear& d, dim3 grid, hipStream_t s, int vecA, int vecW) {
     switch (d.epilogue) {
         case I64H_EPI_GELU_MUL: hipLaunchKernelGGL((linear_tile_kernel<EXACT, I64H_EPI_GELU_MUL>), grid, dim3(256), 0, s, d, vecA, vecW); break;
+        case I64H_EPI_SILU_MUL: hipLaunchKernelGGL((linear_tile_kernel<EXACT, I64H_EPI_SILU_MUL>), grid, dim3(256), 0, s, d, vecA, vecW); break;
         case I64H_EPI_MUL_SIGMOID: hipLaunchKernelGGL((linear_tile_kernel<EXACT, I64H_EPI_MUL_SIGMOID>), grid, dim3(256), 0, s, d, vecA, vecW); break;
         case I64H_EPI_SOFTCAP: hipLaunchKernelGGL((linear_tile_kernel<EXACT, I64H_EPI_SOFTCAP>), grid, dim3(256), 0, s, d, vecA, vecW); break;
         case I64H_EPI_GELU_ERF: hipLaunchKernelGGL((linear_tile_kernel<EXACT, I64H_EPI_GELU_ERF>), grid, dim3(256), 0, s, d, vecA, vecW); break;
+        case I64H_EPI_XIELU: hipLaunchKernelGGL((linear_tile_kernel<EXACT, I64H_EPI_XIELU>), grid, dim3(256), 0, s, d, vecA, vecW); break;
         case I64H_EPI_SCALE: hipLaunchKernelGGL((linear_tile_kernel<EXACT, I64H_EPI_SCALE>), grid, dim3(256), 0, s, d, vecA, vecW); break;
         default: hipLaunchKernelGGL((linear_tile_kernel<EXACT, I64H_EPI_STORE>), grid, dim3(256), 0, s, d, vecA, vecW); break;
     }
@@ -691,10 +708,10 @@ int i64h_linear_run(const i64h_linear* dp, void* stream) {
     const i64h_linear& d = *dp;
     I64H_CHECK_ARG(d.M >= 0 && d.N > 0 && d.K > 0 && d.batch > 0, "linear: bad sizes M=%lld N=%d K=%d batch=%d", (long long)d.M, d.N, d.K, d.batch);
     I64H_CHECK_ARG(d.A && d.W && d.C, "linear: null operand");
-    I64H_CHECK_ARG(d.epilogue >= 0 && d.epilogue <= 5, "linear: epilogue %d", d.epilogue);
+    I64H_CHECK_ARG(d.epilogue >= 0 && d.epilogue <= 7, "linear: epilogue %d", d.epilogue);
     I64H_CHECK_ARG(d.epilogue != I64H_EPI_MUL_SIGMOID || d.E, "linear: the sigmoid epilogue needs E");
     I64H_CHECK_ARG(d.epilogue != I64H_EPI_SOFTCAP || d.softcap > 0.0f, "linear: soft cap %g", (double)d.softcap);
-    I64H_CHECK_ARG(d.epilogue != I64H_EPI_GELU_MUL || !d.bias, "linear: the gate / up epilogue takes no bias");
+    I64H_CHECK_ARG(!dn_dual(d.epilogue) || !d.bias, "linear: the gate / up epilogues take no bias");
     I64H_CHECK_ARG(d.lda >= d.K || d.M <= 1, "linear: lda %lld < K %d", (long long)d.lda, d.K);
     I64H_CHECK_ARG(d.batch <= 65535 && (d.M + 63) / 64 <= 65535, "linear: grid too large");
     if (d.M == 0) return 0;
@@ -702,29 +719,33 @@ int i64h_linear_run(const i64h_linear* dp, void* stream) {
     const int vecW = (uintptr_t)d.W % 16 == 0 && d.K % 8 == 0 && d.w_batch % 8 == 0;
     hipStream_t s = (hipStream_t)stream;
     const size_t lds = (size_t)d.M * d.K * 2;
-    if (g_skinny && !d.exact && d.M <= I64H_SKINNY_ROWS && vecA && vecW && lds <= 64 * 1024) {
+    if (g_skinny && !d.group_off && !d.exact && d.M <= I64H_SKINNY_ROWS && vecA && vecW && lds <= 64 * 1024) {
         int cpb = 64;  // columns per workgroup: at least about two workgroups per CU, a wave takes four columns at a time
         while (cpb > 16 && (int64_t)((d.N + cpb - 1) / cpb) * d.batch < 512) cpb >>= 1;
         const dim3 grid((unsigned)((d.N + cpb - 1) / cpb), 1, (unsigned)d.batch);
         switch (d.epilogue) {
             case I64H_EPI_GELU_MUL: hipLaunchKernelGGL((linear_skinny_kernel<I64H_EPI_GELU_MUL>), grid, dim3(256), lds, s, d, cpb); break;
+            case I64H_EPI_SILU_MUL: hipLaunchKernelGGL((linear_skinny_kernel<I64H_EPI_SILU_MUL>), grid, dim3(256), lds, s, d, cpb); break;
             case I64H_EPI_MUL_SIGMOID: hipLaunchKernelGGL((linear_skinny_kernel<I64H_EPI_MUL_SIGMOID>), grid, dim3(256), lds, s, d, cpb); break;
             case I64H_EPI_SOFTCAP: hipLaunchKernelGGL((linear_skinny_kernel<I64H_EPI_SOFTCAP>), grid, dim3(256), lds, s, d, cpb); break;
             case I64H_EPI_GELU_ERF: hipLaunchKernelGGL((linear_skinny_kernel<I64H_EPI_GELU_ERF>), grid, dim3(256), lds, s, d, cpb); break;
+            case I64H_EPI_XIELU: hipLaunchKernelGGL((linear_skinny_kernel<I64H_EPI_XIELU>), grid, dim3(256), lds, s, d, cpb); break;
             case I64H_EPI_SCALE: hipLaunchKernelGGL((linear_skinny_kernel<I64H_EPI_SCALE>), grid, dim3(256), lds, s, d, cpb); break;
             default: hipLaunchKernelGGL((linear_skinny_kernel<I64H_EPI_STORE>), grid, dim3(256), lds, s, d, cpb); break;
         }
         I64H_CHECK_LAUNCH();
         return 0;
     }
-    if (g_rows64 && !d.exact && d.M <= 64 && vecA && vecW) {
+    if (g_rows64 && !d.group_off && !d.exact && d.M <= 64 && vecA && vecW) {
         const dim3 grid((unsigned)((d.N + 15) / 16), 1, (unsigned)d.batch);
         switch (d.epilogue) {
             // eight waves share the k steps where one accumulator is kept (the gate / up pair needs twice the LDS: four)
             case I64H_EPI_GELU_MUL: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_GELU_MUL, 4>), grid, dim3(256), 0, s, d); break;
+            case I64H_EPI_SILU_MUL: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_SILU_MUL, 4>), grid, dim3(256), 0, s, d); break;
             case I64H_EPI_MUL_SIGMOID: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_MUL_SIGMOID, 8>), grid, dim3(512), 0, s, d); break;
             case I64H_EPI_SOFTCAP: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_SOFTCAP, 8>), grid, dim3(512), 0, s, d); break;
             case I64H_EPI_GELU_ERF: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_GELU_ERF, 8>), grid, dim3(512), 0, s, d); break;
+            case I64H_EPI_XIELU: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_XIELU, 8>), grid, dim3(512), 0, s, d); break;
             case I64H_EPI_SCALE: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_SCALE, 8>), grid, dim3(512), 0, s, d); break;
             default: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_STORE, 8>), grid, dim3(512), 0, s, d); break;
         }
@@ -732,13 +753,15 @@ int i64h_linear_run(const i64h_linear* dp, void* stream) {
         return 0;
     }
     const int64_t tiles128 = ((d.N + 127) / 128) * ((d.M + 127) / 128) * (int64_t)d.batch;
-    if (g_tile128 && !d.exact && tiles128 >= 256) {     // at least a workgroup per CU: the large tile pays
+    if (g_tile128 && !d.group_off && !d.exact && tiles128 >= 256) {     // at least a workgroup per CU: the large tile pays
         const dim3 grid((unsigned)((d.N + 127) / 128), (unsigned)((d.M + 127) / 128), (unsigned)d.batch);
         switch (d.epilogue) {
             case I64H_EPI_GELU_MUL: hipLaunchKernelGGL((linear_tile128_kernel<I64H_EPI_GELU_MUL>), grid, dim3(256), 0, s, d, vecA, vecW); break;
+            case I64H_EPI_SILU_MUL: hipLaunchKernelGGL((linear_tile128_kernel<I64H_EPI_SILU_MUL>), grid, dim3(256), 0, s, d, vecA, vecW); break;
             case I64H_EPI_MUL_SIGMOID: hipLaunchKernelGGL((linear_tile128_kernel<I64H_EPI_MUL_SIGMOID>), grid, dim3(256), 0, s, d, vecA, vecW); break;
             case I64H_EPI_SOFTCAP: hipLaunchKernelGGL((linear_tile128_kernel<I64H_EPI_SOFTCAP>), grid, dim3(256), 0, s, d, vecA, vecW); break;
             case I64H_EPI_GELU_ERF: hipLaunchKernelGGL((linear_tile128_kernel<I64H_EPI_GELU_ERF>), grid, dim3(256), 0, s, d, vecA, vecW); break;
+            case I64H_EPI_XIELU: hipLaunchKernelGGL((linear_tile128_kernel<I64H_EPI_XIELU>), grid, dim3(256), 0, s, d, vecA, vecW); break;
             case I64H_EPI_SCALE: hipLaunchKernelGGL((linear_tile128_kernel<I64H_EPI_SCALE>), grid, dim3(256), 0, s, d, vecA, vecW); break;
             default: hipLaunchKernelGGL((linear_tile128_kernel<I64H_EPI_STORE>), grid, dim3(256), 0, s, d, vecA, vecW); break;
         }

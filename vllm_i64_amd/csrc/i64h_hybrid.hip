@@ -46,8 +46,10 @@ __global__ __launch_bounds__(256) void embed_bigram_kernel(const i64h_embed_bigr
         }
     }
     const int64_t plane = p.n * (int64_t)W;
+    const int64_t prow = p.pos_table ? min(max((int64_t)p.positions[t], (int64_t)0), p.pos_rows - 1) : 0;
     for (int c = threadIdx.x; c < W; c += 256) {
         float v = hy_bf16(p.table, id * W + c);
+        if (p.pos_table) v += hy_bf16(p.pos_table, prow * W + c);
         if (brow >= 0) v += hy_bf16(p.bigram, brow * W + c);
         for (int s = 0; s < p.copies; ++s) p.out[s * plane + t * W + c] = v;
     }
@@ -83,6 +85,14 @@ __global__ __launch_bounds__(256) void streams_kernel(const i64h_streams_args p)
         b = hy_block_sum(b, red);
         ya = 1.0f / sqrtf(a / (float)W + p.y_eps);
         yb = 1.0f / sqrtf(b / (float)W + p.y_eps);
+    } else if (p.y && p.yn_w) {   // one result with a norm of its own (the norm behind a sublayer)
+        float a = 0.0f;
+        for (int c = tid; c < W; c += 256) {
+            const float u = p.y[m * p.ldy + c];
+            a += u * u;
+        }
+        a = hy_block_sum(a, red);
+        ya = sqrtf(a / (float)W + p.y_eps);     // divided by, as the norm in front is
     }
     float ss = 0.0f;
     for (int c = tid; c < W; c += 256) {
@@ -92,6 +102,7 @@ __global__ __launch_bounds__(256) void streams_kernel(const i64h_streams_args p)
         if (p.y) {
             float v = p.y[m * p.ldy + c];
             if (p.y2) v = 0.5f * (v * ya * p.yn_w[c] + p.y2[m * p.ldy2 + c] * yb * p.y2n_w[c]);
+            else if (p.yn_w) v = v / ya * p.yn_w[c];
             float nx[HY_MAX_STREAMS];
 #pragma unroll
             for (int t = 0; t < HY_MAX_STREAMS; ++t) {
@@ -145,8 +156,9 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(const i64h_causal_conv
     const int before = conv_rows_before(p, t);
     float a = p.bias ? p.bias[c] : 0.0f;
     for (int k = 0; k < p.taps - 1; ++k) a += p.w[(int64_t)c * p.taps + k] * conv_input(p, t, p.taps - 1 - k, before, c);
-    a += p.w[(int64_t)c * p.taps + p.taps - 1] * p.P[t * p.ldp + p.off + c];
-    p.out[t * p.ldo + c] = hy_silu(a);
+    const float x = p.P[t * p.ldp + p.off + c];
+    a += p.w[(int64_t)c * p.taps + p.taps - 1] * x;
+    p.out[t * p.ldo + c] = p.mode == 1 ? x + a : hy_silu(a);
 }
 
 // the same for 2 .. 8 taps: a thread walks CV_ROWS consecutive rows of its channel with the weights and the last TAPS - 1 inputs in
@@ -172,7 +184,7 @@ __global__ __launch_bounds__(256) void causal_conv_walk_kernel(const i64h_causal
 #pragma unroll
         for (int k = 0; k < TAPS - 1; ++k) a += w[k] * win[TAPS - 2 - k];
         a += w[TAPS - 1] * x;
-        p.out[t * p.ldo + c] = hy_silu(a);
+        p.out[t * p.ldo + c] = p.mode == 1 ? x + a : hy_silu(a);
 #pragma unroll
         for (int d = TAPS - 2; d > 0; --d) win[d] = win[d - 1];
         win[0] = x;
@@ -432,7 +444,9 @@ __global__ __launch_bounds__(256) void kattn_prep_kernel(const i64h_kattn_prep_a
     if (tid == 0) p.kscale[row] = kr;
 }
 
-// one wave per (row, head): the lanes take 64 keys at a time for the scores, then the value columns for the weighted sum
+// one wave per (row, head): the lanes take 64 keys at a time for the scores, then the value columns for the weighted sum.  With
+// vdim > 0 a key head's part of a cached row is [vdim values | dim key values] and the query sits behind vdim zeros in its Q row;
+// otherwise the dim key values are the values too.
 #define KA_MAX_DIM 256
 template <typename T>
 __global__ __launch_bounds__(256) void kattn_row_kernel(const i64h_kattn_args p) {
@@ -445,11 +459,12 @@ __global__ __launch_bounds__(256) void kattn_row_kernel(const i64h_kattn_args p)
     const int64_t t = item / p.heads;
     const int h = (int)(item % p.heads);
     const int g = h / (p.heads / p.kv_heads);
-    const int dim = p.dim, nk = p.kv_heads * dim;
+    const int dim = p.dim, vd = p.vdim > 0 ? p.vdim : dim, koff = p.vdim > 0 ? p.vdim : 0, gs = koff + dim;
+    const int nk = p.kv_heads * gs;
     const int pos = p.positions[t], slot = p.slot_ids[t];
     const int lo = p.chunk > 0 ? (pos / p.chunk) * p.chunk : 0;
     const T* cache = (const T*)p.cache;
-    for (int d = lane; d < dim; d += 64) sq[wid][d] = p.Q[(t * p.heads + h) * dim + d];
+    for (int d = lane; d < dim; d += 64) sq[wid][d] = p.Q[(t * p.heads + h) * gs + koff + d];
     float m = p.sink ? 0.0f : -INFINITY, l = p.sink ? 1.0f : 0.0f;
     float acc[KA_MAX_DIM / 64] = {0.0f, 0.0f, 0.0f, 0.0f};
     for (int j0 = lo; j0 <= pos; j0 += 64) {
@@ -458,10 +473,10 @@ __global__ __launch_bounds__(256) void kattn_row_kernel(const i64h_kattn_args p)
         int64_t row = 0;
         if (j <= pos) {
             row = cache_row(p.block_table, p.max_blocks_per_seq, p.block_size, slot, j);
-            const T* kr = cache + row * nk + g * dim;
+            const T* kr = cache + row * nk + g * gs + koff;
             float dot = 0.0f;
             for (int d = 0; d < dim; ++d) dot += sq[wid][d] * (float)kr[d];
-            s = dot * p.kscale[row];
+            s = p.kscale ? dot * p.kscale[row] : dot;
             if (p.bias) s += p.bias[(int64_t)min(pos - j, p.bias_rows - 1) * p.heads + h];
         }
         srow[wid][lane] = row;
@@ -475,9 +490,9 @@ __global__ __launch_bounds__(256) void kattn_row_kernel(const i64h_kattn_args p)
 #pragma unroll
         for (int i = 0; i < KA_MAX_DIM / 64; ++i) {
             const int d = lane + 64 * i;
-            if (d < dim) {
+            if (d < vd) {
                 float a = acc[i] * f;
-                for (int u = 0; u < cnt; ++u) a += sp[wid][u] * (float)cache[srow[wid][u] * nk + g * dim + d];
+                for (int u = 0; u < cnt; ++u) a += sp[wid][u] * (float)cache[srow[wid][u] * nk + g * gs + d];
                 acc[i] = a;
             }
         }
@@ -485,7 +500,29 @@ __global__ __launch_bounds__(256) void kattn_row_kernel(const i64h_kattn_args p)
 #pragma unroll
     for (int i = 0; i < KA_MAX_DIM / 64; ++i) {
         const int d = lane + 64 * i;
-        if (d < dim) p.out[(t * p.heads + h) * dim + d] = acc[i] / l;
+        if (d < vd) p.out[(t * p.heads + h) * vd + d] = acc[i] / l;
+    }
+}
+
+// [q | k | v] projections -> the paged cache row [v | k] per key head and the query rows [0 | q * scale]
+__global__ __launch_bounds__(256) void kv_prep_kernel(const i64h_kv_prep_args p) {
+    const int tid = threadIdx.x;
+    const int64_t t = blockIdx.x;
+    const int gs = p.vdim + p.dim;
+    const float* row = p.P + t * p.ldp;
+    float* Q = p.Q + t * p.heads * gs;
+    for (int c = tid; c < p.heads * gs; c += 256) {
+        const int h = c / gs, d = c % gs;
+        Q[c] = d < p.vdim ? 0.0f : row[p.q_off + h * p.dim + d - p.vdim] * p.scale;
+    }
+    if (!p.cache) return;
+    const int64_t cr = cache_row(p.block_table, p.max_blocks_per_seq, p.block_size, p.slot_ids[t], p.positions[t]);
+    const int nk = p.kv_heads * gs;
+    for (int c = tid; c < nk; c += 256) {
+        const int g = c / gs, d = c % gs;
+        const float v = d < p.vdim ? row[p.v_off + g * p.vdim + d] : row[p.k_off + g * p.dim + d - p.vdim];
+        if (p.cache_dtype == 0) ((float*)p.cache)[cr * nk + c] = v;
+        else ((__bf16*)p.cache)[cr * nk + c] = (__bf16)v;
     }
 }
 
@@ -498,6 +535,7 @@ int i64h_embed_bigram(const i64h_embed_bigram_args* dp, void* stream) {
     I64H_CHECK_ARG(d.n >= 0 && d.W > 0 && d.V > 0 && d.copies >= 1, "embed_bigram: bad sizes");
     I64H_CHECK_ARG(d.ids && d.table && d.out && d.positions && d.slot_ids, "embed_bigram: null operand");
     I64H_CHECK_ARG(!d.bigram || (d.buckets > 0 && d.prev_token), "embed_bigram: the bigram table needs buckets and the previous tokens");
+    I64H_CHECK_ARG(!d.pos_table || d.pos_rows > 0, "embed_bigram: an empty position table");
     if (d.n == 0) return 0;
     hipLaunchKernelGGL(embed_bigram_kernel, dim3((unsigned)d.n), dim3(256), 0, (hipStream_t)stream, d);
     I64H_CHECK_LAUNCH();
@@ -532,6 +570,7 @@ int i64h_causal_conv(const i64h_causal_conv_args* dp, void* stream) {
     I64H_CHECK_ARG(d.channels > 0 && d.taps >= 1 && d.taps <= HY_MAX_TAPS && d.n >= 0, "causal_conv: %d channels, %d taps (at most %d)", d.channels, d.taps, HY_MAX_TAPS);
     I64H_CHECK_ARG(d.P && d.w && d.out && d.positions && d.slot_ids && (d.state || d.taps == 1), "causal_conv: null operand");
     I64H_CHECK_ARG(d.n <= 65535, "causal_conv: %lld rows in one launch (at most 65535)", (long long)d.n);
+    I64H_CHECK_ARG(d.mode == 0 || d.mode == 1, "causal_conv: mode %d", d.mode);
     if (d.n == 0) return 0;
     const dim3 grid((unsigned)((d.channels + 255) / 256), (unsigned)d.n);
     const dim3 walk((unsigned)((d.channels + 255) / 256), (unsigned)((d.n + CV_ROWS - 1) / CV_ROWS));
@@ -636,17 +675,21 @@ int i64h_kattn(const i64h_kattn_args* dp, void* stream) {
     const i64h_kattn_args& d = *dp;
     I64H_CHECK_ARG(d.heads > 0 && d.kv_heads > 0 && d.heads % d.kv_heads == 0 && d.dim > 0 && d.dim <= KA_MAX_DIM, "kattn: heads %d, kv heads %d, dim %d (at most %d)",
                    d.heads, d.kv_heads, d.dim, KA_MAX_DIM);
-    I64H_CHECK_ARG(d.Q && d.cache && d.kscale && d.block_table && d.slot_ids && d.positions && d.out, "kattn: null operand");
+    I64H_CHECK_ARG(d.vdim >= 0 && d.vdim <= KA_MAX_DIM, "kattn: vdim %d (at most %d)", d.vdim, KA_MAX_DIM);
+    I64H_CHECK_ARG(d.Q && d.cache && (d.kscale || d.vdim > 0) && d.block_table && d.slot_ids && d.positions && d.out, "kattn: null operand");
     I64H_CHECK_ARG(d.cache_dtype == 0 || d.cache_dtype == 2, "kattn: cache type %d", d.cache_dtype);
     I64H_CHECK_ARG(!d.bias || d.bias_rows > 0, "kattn: an empty bias table");
     I64H_CHECK_ARG(d.block_size > 0 && d.max_blocks_per_seq > 0, "kattn: bad paging");
     if (d.n == 0) return 0;
-    if (d.mode != 1 && d.cache_dtype == 2 && d.dim % 16 == 0 && d.dim <= 256 && (uintptr_t)d.Q % 16 == 0 && (uintptr_t)d.cache % 16 == 0) {
+    // the matrix-core kernel of the latent attention scores against a whole cached row part and sums its first columns: the keys as values
+    // (all columns) or [values | keys] with zeros in the query's value columns
+    const int vals = d.vdim > 0 ? d.vdim : d.dim, gs = d.vdim > 0 ? d.vdim + d.dim : d.dim;
+    if (d.mode != 1 && d.cache_dtype == 2 && vals % 16 == 0 && vals <= 256 && gs % 8 == 0 && gs <= 320 && (uintptr_t)d.Q % 16 == 0 && (uintptr_t)d.cache % 16 == 0) {
         i64h_latent_attn_args a = {};
         a.Q = d.Q, a.cache = d.cache, a.cache_dtype = d.cache_dtype, a.block_table = d.block_table, a.max_blocks_per_seq = d.max_blocks_per_seq;
         a.block_size = d.block_size, a.slot_ids = d.slot_ids, a.positions = d.positions, a.window = 0, a.scale = 1.0f, a.out = d.out, a.n = d.n;
-        a.heads = d.heads, a.kv_rank = d.dim, a.rot_dim = 0, a.mode = d.mode == 3 ? 3 : 2, a.splits = d.splits, a.workspace = d.workspace;
-        a.row_stride = d.kv_heads * d.dim, a.kv_groups = d.kv_heads, a.chunk = d.chunk, a.kscale = d.kscale, a.bias = d.bias, a.bias_rows = d.bias_rows;
+        a.heads = d.heads, a.kv_rank = vals, a.rot_dim = gs - vals, a.mode = d.mode == 3 ? 3 : 2, a.splits = d.splits, a.workspace = d.workspace;
+        a.row_stride = d.kv_heads * gs, a.kv_groups = d.kv_heads, a.chunk = d.chunk, a.kscale = d.kscale, a.bias = d.bias, a.bias_rows = d.bias_rows;
         a.sink = d.sink;
         return i64h_latent_attn(&a, stream);
     }
@@ -654,6 +697,19 @@ int i64h_kattn(const i64h_kattn_args* dp, void* stream) {
     const dim3 grid((unsigned)((items + 3) / 4));
     if (d.cache_dtype == 0) hipLaunchKernelGGL((kattn_row_kernel<float>), grid, dim3(256), 0, (hipStream_t)stream, d);
     else hipLaunchKernelGGL((kattn_row_kernel<__bf16>), grid, dim3(256), 0, (hipStream_t)stream, d);
+    I64H_CHECK_LAUNCH();
+    return 0;
+}
+
+int i64h_kv_prep(const i64h_kv_prep_args* dp, void* stream) {
+    I64H_CHECK_ARG(dp != nullptr, "kv_prep: no descriptor");
+    const i64h_kv_prep_args& d = *dp;
+    I64H_CHECK_ARG(d.heads > 0 && d.kv_heads > 0 && d.heads % d.kv_heads == 0 && d.dim > 0 && d.vdim > 0, "kv_prep: heads %d, kv heads %d, dim %d, vdim %d",
+                   d.heads, d.kv_heads, d.dim, d.vdim);
+    I64H_CHECK_ARG(d.P && d.Q && d.positions && d.slot_ids, "kv_prep: null operand");
+    I64H_CHECK_ARG(!d.cache || (d.block_table && d.block_size > 0 && d.max_blocks_per_seq > 0 && (d.cache_dtype == 0 || d.cache_dtype == 2)), "kv_prep: bad paging or cache type");
+    if (d.n == 0) return 0;
+    hipLaunchKernelGGL(kv_prep_kernel, dim3((unsigned)d.n), dim3(256), 0, (hipStream_t)stream, d);
     I64H_CHECK_LAUNCH();
     return 0;
 }

@@ -11,7 +11,8 @@ from . import _lib
 from ._lib import call_dense, ptr
 from .ops import _chk, _stream
 
-EPI_STORE, EPI_GELU_MUL, EPI_MUL_SIGMOID, EPI_SOFTCAP, EPI_GELU_ERF, EPI_SCALE = 0, 1, 2, 3, 4, 5
+EPI_STORE, EPI_GELU_MUL, EPI_MUL_SIGMOID, EPI_SOFTCAP, EPI_GELU_ERF, EPI_SCALE, EPI_SILU_MUL, EPI_XIELU = 0, 1, 2, 3, 4, 5, 6, 7
+_DUAL = (EPI_GELU_MUL, EPI_SILU_MUL)
 CACHE_DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 2}
 
 
@@ -23,14 +24,17 @@ def linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, m: Optional[i
            a_off: int = 0, lda: Optional[int] = None, a_rows: Optional[torch.Tensor] = None, c_off: int = 0, ldc: Optional[int] = None,
            batch: int = 1, a_batch: int = 0, w_batch: int = 0, c_batch: int = 0, exact: bool = False, epilogue: int = EPI_STORE,
            e: Optional[torch.Tensor] = None, e_off: int = 0, lde: int = 0, e_batch: int = 0, softcap: float = 0.0,
-           bias: Optional[torch.Tensor] = None, bias_batch: int = 0, scale: float = 1.0) -> torch.Tensor:
+           bias: Optional[torch.Tensor] = None, bias_batch: int = 0, scale: float = 1.0, act_a: float = 0.0, act_b: float = 0.0,
+           group_off: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[b][:, c_off + b * c_batch : + n] = epilogue(a[b][rows, a_off + b * a_batch : + k] @ w[b]^T): see i64h_linear.  a, out and e are
-    fp32 matrices addressed by (column offset, row stride); w is bf16 [n, k] (EPI_GELU_MUL: [2n, k], gate rows first), or a stack
-    [batch, n, k] with w_batch = n * k.  bias fp32 [n] (per batch: bias_batch apart) is added before the epilogue."""
+    fp32 matrices addressed by (column offset, row stride); w is bf16 [n, k] (EPI_GELU_MUL / EPI_SILU_MUL: [2n, k], gate rows first), or a
+    stack [batch, n, k] with w_batch = n * k.  bias fp32 [n] (per batch: bias_batch apart) is added before the epilogue.  group_off int32
+    [batch + 1] on the device: batch b takes the rows [group_off[b], group_off[b + 1]) of a_rows (or a) and out; m is then the most rows a
+    batch may have, and a_rows / a / out must hold group_off[batch] rows (the caller's business: the counts stay on the device)."""
     _chk(a, torch.float32, "a"), _chk(w, torch.bfloat16, "w"), _chk(out, torch.float32, "out")
     if a_rows is not None:
         _chk(a_rows, torch.int32, "a_rows")
-    N = int(n if n is not None else w.shape[-2] // (2 if epilogue == EPI_GELU_MUL else 1))
+    N = int(n if n is not None else w.shape[-2] // (2 if epilogue in _DUAL else 1))
     K = int(k if k is not None else w.shape[-1])
     M = int(m if m is not None else (a_rows.numel() if a_rows is not None else a.shape[0]))
     lda = int(lda if lda is not None else a.shape[-1])
@@ -39,7 +43,7 @@ def linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, m: Optional[i
         raise _lib.I64HError(f"linear: K {K} / N {N} do not fit a (row stride {lda}), w {tuple(w.shape)} or out (row stride {ldc})")
     if out.numel() < (M - 1) * ldc + c_off + (batch - 1) * c_batch + N or (a_rows is None and a.numel() < (M - 1) * lda + a_off + (batch - 1) * a_batch + K):
         raise _lib.I64HError("linear: operand smaller than the launch reads or writes")
-    if w.numel() < (batch - 1) * w_batch + N * K * (2 if epilogue == EPI_GELU_MUL else 1):
+    if w.numel() < (batch - 1) * w_batch + N * K * (2 if epilogue in _DUAL else 1):
         raise _lib.I64HError("linear: weight smaller than the launch reads")
     if e is not None:
         _chk(e, torch.float32, "e")
@@ -49,10 +53,14 @@ def linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, m: Optional[i
         _chk(bias, torch.float32, "bias")
         if bias.numel() < (batch - 1) * bias_batch + N:
             raise _lib.I64HError("linear: bias smaller than the launch reads")
+    if group_off is not None:
+        _chk(group_off, torch.int32, "group_off")
+        if group_off.numel() < batch + 1:
+            raise _lib.I64HError("linear: group_off needs batch + 1 entries")
     d = _lib.Linear(A=ptr(a) + 4 * a_off, lda=lda, a_rows=ptr(a_rows), W=ptr(w), C=ptr(out) + 4 * c_off, ldc=ldc, M=M, N=N, K=K, batch=batch,
                     a_batch=a_batch, w_batch=w_batch, c_batch=c_batch, exact=int(exact), epilogue=epilogue,
                     E=(ptr(e) + 4 * e_off) if e is not None else 0, lde=lde, e_batch=e_batch, softcap=float(softcap),
-                    bias=ptr(bias), bias_batch=int(bias_batch), scale=float(scale))
+                    bias=ptr(bias), bias_batch=int(bias_batch), scale=float(scale), act_a=float(act_a), act_b=float(act_b), group_off=ptr(group_off))
     call_dense("i64h_linear_run", _ref(d), _stream())
     return out
 
@@ -148,8 +156,8 @@ def _rows_ok(name: str, n: int, *tensors) -> None:
 
 def embed_bigram(ids: torch.Tensor, positions: torch.Tensor, slot_ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, *,
                  bigram: Optional[torch.Tensor] = None, buckets: int = 0, mul_prev: int = 0, mul_cur: int = 0,
-                 prev_token: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """See i64h_embed_bigram.  out fp32 [copies, n, W] (or [n, W]); prev_token int64 [slots], read and updated."""
+                 prev_token: Optional[torch.Tensor] = None, pos_table: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """See i64h_embed_bigram.  out fp32 [copies, n, W] (or [n, W]); prev_token int64 [slots], read and updated; pos_table bf16 [positions, W]."""
     _chk(ids, torch.int64, "ids"), _chk(positions, torch.int32, "positions"), _chk(slot_ids, torch.int32, "slot_ids")
     _chk(table, torch.bfloat16, "table"), _chk(out, torch.float32, "out")
     n = ids.numel()
@@ -162,9 +170,13 @@ def embed_bigram(ids: torch.Tensor, positions: torch.Tensor, slot_ids: torch.Ten
         _chk(bigram, torch.bfloat16, "bigram"), _chk(prev_token, torch.int64, "prev_token")
         if tuple(bigram.shape) != (buckets + 1, W):
             raise _lib.I64HError(f"embed_bigram: table {tuple(bigram.shape)} for {buckets} buckets of width {W}")
+    if pos_table is not None:
+        _chk(pos_table, torch.bfloat16, "pos_table")
+        if pos_table.dim() != 2 or pos_table.shape[1] != W:
+            raise _lib.I64HError(f"embed_bigram: position table {tuple(pos_table.shape)} for width {W}")
     d = _lib.EmbedBigram(ids=ptr(ids), positions=ptr(positions), slot_ids=ptr(slot_ids), table=ptr(table), V=V, W=W, bigram=ptr(bigram),
                          buckets=int(buckets), mul_prev=int(mul_prev), mul_cur=int(mul_cur), prev_token=ptr(prev_token), out=ptr(out),
-                         copies=max(1, copies), n=n)
+                         copies=max(1, copies), n=n, pos_table=ptr(pos_table), pos_rows=pos_table.shape[0] if pos_table is not None else 0)
     call_dense("i64h_embed_bigram", _ref(d), _stream())
     return out
 
@@ -200,20 +212,26 @@ def streams_step(streams: torch.Tensor, *, y: Optional[torch.Tensor] = None, y2:
 
 
 def causal_conv(p: torch.Tensor, *, off: int, channels: int, w: torch.Tensor, bias: Optional[torch.Tensor], positions: torch.Tensor,
-                slot_ids: torch.Tensor, state: torch.Tensor, out: torch.Tensor, n: Optional[int] = None) -> torch.Tensor:
-    """See i64h_causal_conv.  p fp32 [n, ldp]; w fp32 [channels, taps]; state fp32 [slots, taps - 1, channels]; out fp32 [n, channels]."""
-    _chk(p, torch.float32, "p"), _chk(w, torch.float32, "w"), _chk(state, torch.float32, "state"), _chk(out, torch.float32, "out")
+                slot_ids: torch.Tensor, state: Optional[torch.Tensor], out: torch.Tensor, n: Optional[int] = None, added: bool = False) -> torch.Tensor:
+    """See i64h_causal_conv.  p fp32 [n, ldp]; w fp32 [channels, taps]; state fp32 [slots, taps - 1, channels]; out fp32 [n, channels].
+    added: the convolution is added to its own input and no activation follows (mode 1)."""
+    _chk(p, torch.float32, "p"), _chk(w, torch.float32, "w"), _chk(out, torch.float32, "out")
     _chk(positions, torch.int32, "positions"), _chk(slot_ids, torch.int32, "slot_ids")
     rows = int(n if n is not None else positions.numel())
     taps = w.shape[-1]
+    if state is None:
+        if taps > 1:
+            raise _lib.I64HError("causal_conv: more than one tap needs the carried inputs")
+        state = out      # (never read or written with one tap)
+    _chk(state, torch.float32, "state")
     _rows_ok("causal_conv", rows, positions, slot_ids)
     if bias is not None:
         _chk(bias, torch.float32, "bias")
     if w.shape[0] != channels or off + channels > p.shape[-1] or p.numel() < rows * p.shape[-1] or out.numel() < rows * channels or \
-            (bias is not None and bias.numel() != channels) or state.shape[-1] != channels or state.shape[-2] != max(taps - 1, 0):
+            (bias is not None and bias.numel() != channels) or (taps > 1 and (state.shape[-1] != channels or state.shape[-2] != taps - 1)):
         raise _lib.I64HError("causal_conv: shapes do not fit the sizes")
     d = _lib.CausalConv(P=ptr(p), ldp=p.shape[-1], off=off, channels=channels, taps=taps, w=ptr(w), bias=ptr(bias), positions=ptr(positions),
-                        slot_ids=ptr(slot_ids), state=ptr(state), out=ptr(out), ldo=channels, n=rows)
+                        slot_ids=ptr(slot_ids), state=ptr(state), out=ptr(out), ldo=channels, n=rows, mode=1 if added else 0)
     call_dense("i64h_causal_conv", _ref(d), _stream())
     return out
 
@@ -295,9 +313,12 @@ def kattn_prep(p: torch.Tensor, *, q_off: int, k_off: int, heads: int, kv_heads:
 
 def kattn(q: torch.Tensor, cache: torch.Tensor, kscale: torch.Tensor, block_table: torch.Tensor, slot_ids: torch.Tensor, positions: torch.Tensor, *,
           chunk: int, bias: Optional[torch.Tensor], sink: bool, heads: int, kv_heads: int, dim: int, out: torch.Tensor, n: Optional[int] = None,
-          mode: int = 0, splits: int = 1, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """See i64h_kattn.  q, out fp32 [n, heads * dim]; bias fp32 [distances, heads]."""
-    _chk(q, torch.float32, "q"), _chk(out, torch.float32, "out"), _chk(cache, None, "cache"), _chk(kscale, torch.float32, "kscale")
+          mode: int = 0, splits: int = 1, workspace: Optional[torch.Tensor] = None, vdim: int = 0) -> torch.Tensor:
+    """See i64h_kattn.  q, out fp32 [n, heads * dim]; bias fp32 [distances, heads].  vdim > 0: separate values - the cache rows are
+    [kv_heads, vdim + dim], q fp32 [n, heads, vdim + dim], out fp32 [n, heads * vdim], kscale may be None."""
+    _chk(q, torch.float32, "q"), _chk(out, torch.float32, "out"), _chk(cache, None, "cache")
+    if kscale is not None or vdim <= 0:
+        _chk(kscale, torch.float32, "kscale")
     _chk(positions, torch.int32, "positions"), _chk(slot_ids, torch.int32, "slot_ids"), _chk(block_table, torch.int32, "block_table")
     rows = int(n if n is not None else positions.numel())
     _rows_ok("kattn", rows, positions, slot_ids)
@@ -305,10 +326,12 @@ def kattn(q: torch.Tensor, cache: torch.Tensor, kscale: torch.Tensor, block_tabl
         _chk(bias, torch.float32, "bias")
         if bias.dim() != 2 or bias.shape[1] != heads:
             raise _lib.I64HError("kattn: bias is not [distances, heads]")
-    if cache.shape[-1] != kv_heads * dim or kscale.numel() != cache.shape[0] * cache.shape[1] or q.numel() < rows * heads * dim or out.numel() < rows * heads * dim:
+    gs, vals = (vdim + dim, vdim) if vdim > 0 else (dim, dim)
+    if cache.shape[-1] != kv_heads * gs or (kscale is not None and kscale.numel() != cache.shape[0] * cache.shape[1]) or q.numel() < rows * heads * gs or \
+            out.numel() < rows * heads * vals:
         raise _lib.I64HError("kattn: shapes do not fit the sizes")
     if splits > 1:
-        need = kattn_workspace_floats(rows, heads, kv_heads, dim, splits)
+        need = kattn_workspace_floats(rows, heads, kv_heads, vals, splits)
         if workspace is None:
             workspace = torch.empty(need, dtype=torch.float32, device=q.device)
         _chk(workspace, torch.float32, "workspace")
@@ -317,13 +340,112 @@ def kattn(q: torch.Tensor, cache: torch.Tensor, kscale: torch.Tensor, block_tabl
     d = _lib.KAttn(Q=ptr(q), cache=ptr(cache), cache_dtype=CACHE_DTYPE_CODE[cache.dtype], kscale=ptr(kscale), block_table=ptr(block_table),
                    max_blocks_per_seq=block_table.shape[1], block_size=cache.shape[-2], slot_ids=ptr(slot_ids), positions=ptr(positions), chunk=int(chunk),
                    bias=ptr(bias), bias_rows=bias.shape[0] if bias is not None else 0, sink=int(bool(sink)), out=ptr(out), n=rows, heads=heads,
-                   kv_heads=kv_heads, dim=dim, mode=int(mode), splits=int(splits) if splits > 1 else 1, workspace=ptr(workspace) if splits > 1 else 0)
+                   kv_heads=kv_heads, dim=dim, mode=int(mode), splits=int(splits) if splits > 1 else 1, workspace=ptr(workspace) if splits > 1 else 0,
+                   vdim=int(vdim))
     call_dense("i64h_kattn", _ref(d), _stream())
     return out
 
 
 def kattn_workspace_floats(n: int, heads: int, kv_heads: int, dim: int, splits: int) -> int:
     return int(_lib.load_dense().i64h_kattn_workspace_floats(n, heads, kv_heads, dim, splits))
+
+
+def kv_prep(p: torch.Tensor, *, q_off: int, k_off: int, v_off: int, heads: int, kv_heads: int, dim: int, vdim: int, scale: float, positions: torch.Tensor,
+            slot_ids: torch.Tensor, block_table: torch.Tensor, cache: Optional[torch.Tensor], q: torch.Tensor, n: Optional[int] = None,
+            block_size: int = 0) -> None:
+    """See i64h_kv_prep.  cache [blocks, block, kv_heads * (vdim + dim)] fp32 / bf16 or None (queries only: the rows are another layer's);
+    q fp32 [n, heads, vdim + dim]."""
+    _chk(p, torch.float32, "p"), _chk(q, torch.float32, "q")
+    _chk(positions, torch.int32, "positions"), _chk(slot_ids, torch.int32, "slot_ids"), _chk(block_table, torch.int32, "block_table")
+    rows = int(n if n is not None else positions.numel())
+    _rows_ok("kv_prep", rows, positions, slot_ids)
+    gs = vdim + dim
+    if q.numel() < rows * heads * gs or q_off + heads * dim > p.shape[-1] or p.numel() < rows * p.shape[-1]:
+        raise _lib.I64HError("kv_prep: shapes do not fit the sizes")
+    if cache is not None:
+        _chk(cache, None, "cache")
+        if cache.shape[-1] != kv_heads * gs or max(k_off + kv_heads * dim, v_off + kv_heads * vdim) > p.shape[-1]:
+            raise _lib.I64HError("kv_prep: cache rows or projection columns do not fit the sizes")
+    d = _lib.KvPrep(P=ptr(p), ldp=p.shape[-1], q_off=q_off, k_off=k_off, v_off=v_off, heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, scale=float(scale),
+                    positions=ptr(positions), slot_ids=ptr(slot_ids), block_table=ptr(block_table), max_blocks_per_seq=block_table.shape[1],
+                    block_size=cache.shape[-2] if cache is not None else int(block_size), cache=ptr(cache),
+                    cache_dtype=CACHE_DTYPE_CODE[cache.dtype] if cache is not None else 0, Q=ptr(q), n=rows)
+    call_dense("i64h_kv_prep", _ref(d), _stream())
+
+
+def _gla_args(p: torch.Tensor, *, q_off: int, f_off: int, v_off: int, heads: int, dim: int, vdim: int, k_off: int = -1, lower: Optional[torch.Tensor] = None,
+              q_act: bool = False, n: int, **rest) -> "_lib.Gla":
+    _chk(p, torch.float32, "p")
+    if lower is not None:
+        _chk(lower, torch.float32, "lower")
+        if lower.numel() != heads * dim:
+            raise _lib.I64HError("gla: the gate's lower bounds are not [heads * dim]")
+    ld = p.shape[-1]
+    if max(q_off, f_off, max(k_off, 0)) + heads * dim > ld or v_off + heads * vdim > ld or p.numel() < n * ld:
+        raise _lib.I64HError("gla: projection columns outside the projection rows")
+    return _lib.Gla(P=ptr(p), ldp=ld, q_off=q_off, f_off=f_off, k_off=k_off, v_off=v_off, heads=heads, dim=dim, vdim=vdim, lower=ptr(lower),
+                    q_act=int(bool(q_act)), n=n, **rest)
+
+
+def gla_gates(p: torch.Tensor, *, q_off: int, f_off: int, v_off: int, heads: int, dim: int, vdim: int, lower: Optional[torch.Tensor], q_act: bool,
+              n: int) -> None:
+    """See i64h_gla_gates: q <- silu(q) (q_act), f <- lower + (1 - lower) * sigmoid(f), in place on the projection rows p fp32 [n, ldp]."""
+    d = _gla_args(p, q_off=q_off, f_off=f_off, v_off=v_off, heads=heads, dim=dim, vdim=vdim, lower=lower, q_act=q_act, n=n)
+    call_dense("i64h_gla_gates", _ref(d), _stream())
+
+
+def gla_scan(p: torch.Tensor, *, q_off: int, f_off: int, v_off: int, heads: int, dim: int, vdim: int, seg_start: torch.Tensor, nseg: int,
+             positions: torch.Tensor, slot_ids: torch.Tensor, state: torch.Tensor, out: torch.Tensor, n: int, k_off: int = -1) -> torch.Tensor:
+    """See i64h_gla_scan.  state fp32 [slots, heads, vdim, dim]; out fp32 [n, heads * vdim]; k_off < 0: the key is one minus the decay."""
+    _chk(state, torch.float32, "state"), _chk(out, torch.float32, "out")
+    _chk(seg_start, torch.int32, "seg_start"), _chk(positions, torch.int32, "positions"), _chk(slot_ids, torch.int32, "slot_ids")
+    _rows_ok("gla_scan", n, positions, slot_ids)
+    if tuple(state.shape[1:]) != (heads, vdim, dim) or out.numel() < n * heads * vdim or seg_start.numel() < nseg + 1:
+        raise _lib.I64HError("gla_scan: shapes do not fit the sizes")
+    d = _gla_args(p, q_off=q_off, f_off=f_off, v_off=v_off, heads=heads, dim=dim, vdim=vdim, k_off=k_off, n=n, seg_start=ptr(seg_start), nseg=nseg,
+                  positions=ptr(positions), slot_ids=ptr(slot_ids), state=ptr(state), out=ptr(out), ldo=heads * vdim)
+    call_dense("i64h_gla_scan", _ref(d), _stream())
+    return out
+
+
+def route_topk(logits: torch.Tensor, *, entries: int, correction: Optional[torch.Tensor], groups: int, keep: int, top: int, scale: float, idx: torch.Tensor,
+               wgt: torch.Tensor, n: Optional[int] = None) -> None:
+    """See i64h_route_topk.  logits fp32 [n, ld >= entries]; idx int32 [n, top]; wgt fp32 [n, top]."""
+    _chk(logits, torch.float32, "logits"), _chk(idx, torch.int32, "idx"), _chk(wgt, torch.float32, "wgt")
+    rows = int(n if n is not None else logits.shape[0])
+    if correction is not None:
+        _chk(correction, torch.float32, "correction")
+        if correction.numel() != entries:
+            raise _lib.I64HError("route_topk: the correction is not [entries]")
+    if logits.shape[-1] < entries or logits.numel() < rows * logits.shape[-1] or idx.numel() < rows * top or wgt.numel() < rows * top:
+        raise _lib.I64HError("route_topk: shapes do not fit the sizes")
+    d = _lib.Route(logits=ptr(logits), ld=logits.shape[-1], E=entries, correction=ptr(correction), groups=int(groups), keep=int(keep), top=int(top),
+                   scale=float(scale), idx=ptr(idx), wgt=ptr(wgt), n=rows)
+    call_dense("i64h_route_topk", _ref(d), _stream())
+
+
+def moe_plan(idx: torch.Tensor, *, n: int, top: int, experts: int, group_off: torch.Tensor, pair_token: torch.Tensor, pair_row: torch.Tensor) -> None:
+    """See i64h_moe_plan."""
+    for t, name in ((idx, "idx"), (group_off, "group_off"), (pair_token, "pair_token"), (pair_row, "pair_row")):
+        _chk(t, torch.int32, name)
+    if idx.numel() < n * top or group_off.numel() < experts + 1 or pair_token.numel() < n * top or pair_row.numel() < n * top:
+        raise _lib.I64HError("moe_plan: shapes do not fit the sizes")
+    d = _lib.MoePlan(idx=ptr(idx), n=n, top=top, experts=experts, group_off=ptr(group_off), pair_token=ptr(pair_token), pair_row=ptr(pair_row))
+    call_dense("i64h_moe_plan", _ref(d), _stream())
+
+
+def moe_combine(y: torch.Tensor, pair_row: torch.Tensor, wgt: torch.Tensor, h: torch.Tensor, shared: Optional[torch.Tensor], out: torch.Tensor, *,
+                n: int, top: int, width: int) -> torch.Tensor:
+    """See i64h_moe_combine.  y fp32 [pairs, width]; h, shared, out fp32 [n, width]."""
+    _chk(y, torch.float32, "y"), _chk(pair_row, torch.int32, "pair_row"), _chk(wgt, torch.float32, "wgt"), _chk(h, torch.float32, "h"), _chk(out, torch.float32, "out")
+    if shared is not None:
+        _chk(shared, torch.float32, "shared")
+    if min(h.numel(), out.numel(), shared.numel() if shared is not None else out.numel()) < n * width or min(pair_row.numel(), wgt.numel()) < n * top or \
+            y.numel() < n * top * width:
+        raise _lib.I64HError("moe_combine: shapes do not fit the sizes")
+    d = _lib.MoeCombine(Y=ptr(y), pair_row=ptr(pair_row), wgt=ptr(wgt), h=ptr(h), shared=ptr(shared), out=ptr(out), n=n, top=top, W=width)
+    call_dense("i64h_moe_combine", _ref(d), _stream())
+    return out
 
 
 def sample_rows(logits: torch.Tensor, out: Optional[torch.Tensor] = None, temperature: Optional[torch.Tensor] = None,

@@ -78,19 +78,32 @@ class HybridCache(PagePool):
     """Cache of a model whose layers keep different things: pages of key rows for attention layers (one row per token, which is also
     the value, and the reciprocal root mean square of that row as a separate fp32 number), and per-slot state for recurrent layers
     (fp32, one entry per sequence, overwritten by every step).  specs[l] = {"rows": width} and / or {"state": {name: shape}};
+    "kscale": False leaves the per-token number out (rows that hold keys and values as they are); {"rows_of": j} makes layer l read the
+    rows of the earlier layer j (a layer that attends over another layer's keys and values holds none of its own).
     seq_state: per-slot state of the model as a whole, {name: (shape, dtype)}.  Recurrent state needs no clearing when a slot is used
-    again: the kernels take it as empty for a row at position 0."""
+    again: the kernels take it as empty for a row at position 0.  position_limit > 0 bounds a sequence's length (a model with a table
+    of positions)."""
 
-    def __init__(self, specs: Sequence[dict], num_blocks: int, max_seqs: int, device, dtype=torch.bfloat16, block: int = 16, seq_state=None):
-        super().__init__(num_blocks, block, max_seqs, max(1, num_blocks), device)
+    def __init__(self, specs: Sequence[dict], num_blocks: int, max_seqs: int, device, dtype=torch.bfloat16, block: int = 16, seq_state=None,
+                 position_limit: int = 0):
+        per_seq = max(1, num_blocks) if position_limit <= 0 else max(1, min(num_blocks, (position_limit + block - 1) // block))
+        super().__init__(num_blocks, block, max_seqs, per_seq, device, position_limit=position_limit)
         self.dtype = dtype
         self.rows: List = []
         self.kscale: List = []
         self.state: List[Dict[str, torch.Tensor]] = []
         for sp in specs:
+            if sp.get("rows_of") is not None:
+                j = int(sp["rows_of"])
+                if not 0 <= j < len(self.rows) or self.rows[j] is None:
+                    raise ValueError(f"layer {len(self.rows)} reads the rows of layer {j}, which has none")
+                self.rows.append(self.rows[j])
+                self.kscale.append(self.kscale[j])
+                self.state.append({k: torch.zeros((max_seqs, *shape), dtype=torch.float32, device=device) for k, shape in (sp.get("state") or {}).items()})
+                continue
             w = int(sp.get("rows", 0))
             self.rows.append(torch.zeros((num_blocks, block, w), dtype=dtype, device=device) if w else None)
-            self.kscale.append(torch.zeros((num_blocks, block), dtype=torch.float32, device=device) if w else None)
+            self.kscale.append(torch.zeros((num_blocks, block), dtype=torch.float32, device=device) if w and sp.get("kscale", True) else None)
             self.state.append({k: torch.zeros((max_seqs, *shape), dtype=torch.float32, device=device) for k, shape in (sp.get("state") or {}).items()})
         self.seq_state = {k: torch.zeros((max_seqs, *shape), dtype=dt, device=device) for k, (shape, dt) in (seq_state or {}).items()}
 

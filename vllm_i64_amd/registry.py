@@ -44,6 +44,14 @@ def _load_dogalorn(config: dict, tensors, *, device, dtype, max_seqs, max_tokens
     return DogalornModel(cfg, tensors, device=device, dtype=dtype, max_seqs=max_seqs, num_kv_blocks=blocks, kv_block=kv_block)
 
 
+def _load_zabutar(config: dict, tensors, *, device, dtype, max_seqs, max_tokens, kv_block=16, **_):
+    from .config import ZabutarConfig
+    from .zabutar import ZabutarModel
+    cfg = ZabutarConfig.from_dict(config)
+    blocks = max(1, (int(max_tokens) + kv_block - 1) // kv_block)
+    return ZabutarModel(cfg, tensors, device=device, dtype=dtype, max_seqs=max_seqs, num_kv_blocks=blocks, kv_block=kv_block)
+
+
 def _load_complexity_deep(config: dict, tensors, *, device, dtype, max_seqs, max_tokens, quant="int8", **_):
     import torch
     from .checkpoint import config_from_dict, native_to_weights
@@ -56,6 +64,7 @@ def _load_complexity_deep(config: dict, tensors, *, device, dtype, max_seqs, max
 
 register("Morilorn", _load_morilorn)
 register("Dogalorn", _load_dogalorn)
+register("Zabutar", _load_zabutar)
 register("complexity-deep", _load_complexity_deep)
 register("ComplexityDeepModel", _load_complexity_deep)
 
