@@ -129,10 +129,19 @@ def route(z: torch.Tensor, correction: torch.Tensor, r: dict):
     return idx, wgt / (wgt.sum(-1, keepdim=True) + 1e-20) * float(r.get("scale", 1.0))
 
 
-def mixture_ff(W: Dict[str, torch.Tensor], p: str, f: dict, h: torch.Tensor) -> torch.Tensor:
+def mixture_ff(W: Dict[str, torch.Tensor], p: str, f: dict, h: torch.Tensor, forced: Optional[torch.Tensor] = None, chosen: Optional[list] = None) -> torch.Tensor:
+    """forced [T, top]: entries to use instead of the router's own choice (their weights still come from the router's scores) - for
+    comparisons with an implementation in lower precision, where a close call may fall the other way; chosen receives the choice."""
     r = f["router"]
     E = int(r["experts"])
-    idx, wgt = route(h @ W[p + "router"].T, W[p + "correction"], r)
+    z = h @ W[p + "router"].T
+    idx, wgt = route(z, W[p + "correction"], r)
+    if forced is not None:
+        idx = forced.to(torch.int64)
+        wgt = torch.softmax(z, -1).gather(1, idx)
+        wgt = wgt / (wgt.sum(-1, keepdim=True) + 1e-20) * float(r.get("scale", 1.0))
+    if chosen is not None:
+        chosen.append(idx)
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         for e, g in zip(idx[t].tolist(), wgt[t]):
@@ -143,8 +152,10 @@ def mixture_ff(W: Dict[str, torch.Tensor], p: str, f: dict, h: torch.Tensor) -> 
 
 
 # ---- the whole model ---------------------------------------------------------------------------------------------------------------
-def forward(cfg: dict, W32: Dict[str, torch.Tensor], tokens: List[int], record: Optional[list] = None) -> torch.Tensor:
-    """Logits [T, vocab] of one sequence; record (a list) receives the residual after every layer."""
+def forward(cfg: dict, W32: Dict[str, torch.Tensor], tokens: List[int], record: Optional[list] = None, routes: Optional[dict] = None,
+            chosen: Optional[dict] = None) -> torch.Tensor:
+    """Logits [T, vocab] of one sequence; record (a list) receives the residual after every layer; routes: layer -> entries [T, top] to
+    use instead of the router's choice; chosen (a dict) receives every mixture layer's choice."""
     W = {k: v.to(F64) for k, v in W32.items()}
     eps = float(cfg["norm"]["eps"])
     x = embedding(W, tokens)
@@ -165,7 +176,13 @@ def forward(cfg: dict, W32: Dict[str, torch.Tensor], tokens: List[int], record: 
         f = L.get("mlp")
         if f:
             h = input_convolution(W[p + "canon2"], offset_norm(x, W[p + "norm2"], eps))
-            y = dense_ff(W, p + "mlp.", h) if f.get("kind", "dense") == "dense" else mixture_ff(W, p + "mlp.", f, h)
+            if f.get("kind", "dense") == "dense":
+                y = dense_ff(W, p + "mlp.", h)
+            else:
+                got = []
+                y = mixture_ff(W, p + "mlp.", f, h, forced=(routes or {}).get(i), chosen=got)
+                if chosen is not None:
+                    chosen[i] = got[0]
             x = x + offset_norm(y, W[p + "norm2b"], eps)
         if record is not None:
             record.append(x.clone())

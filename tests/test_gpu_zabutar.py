@@ -1,0 +1,663 @@
+"""The Zabutar design on the GPU against the CPU oracle (oracle/zabutar_ref.py): every mechanism alone, then whole models of several
+small shapes under every way of cutting, batching, paging and slotting their sequences, through the engine and the command line.
+Weights are random and bf16-representable; where random weights would hide a fault (a far key among many, a bucket's edge, a state
+that has to last) the inputs are made so that it shows."""
+import json
+import math
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+from oracle import zabutar_ref as R
+from tests.zabutar_shapes import SHAPES, config_of, make_weights, tokens
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+# rms over the vocabulary of the logit difference / rms of the logits, worst position.  bfloat16: the 2^-9 input rounding of every matrix
+# product, carried on by the recurrences, gives about a percent; a wrong mechanism gives 50 % and more.  A router decision that is a close
+# call can fall the other way in bfloat16 and stays in the recurrent state and the cached keys from then on, so the bfloat16 model is
+# compared with the oracle under the model's OWN choices (which must be the oracle's for most tokens), and cuts and batches with the
+# model's own whole prompt.
+TOL = {"float32": 3e-5, "bfloat16": 8e-2}
+
+
+@pytest.fixture(scope="module")
+def dev():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    return torch.device("cuda:0")
+
+
+def row_err(got, want):
+    got, want = torch.as_tensor(got, dtype=torch.float64).cpu(), torch.as_tensor(want, dtype=torch.float64).cpu()
+    d = got - want
+    d = d - d.mean(-1, keepdim=True)
+    return d.pow(2).mean(-1).sqrt() / want.pow(2).mean(-1).sqrt().clamp_min(1e-9)
+
+
+def agrees(got, want, dtype):
+    return float(row_err(got, want).max()) < TOL[dtype]
+
+
+def same_to_rounding(got, want, dtype):
+    """Two runs of the same model that differ in how the sequence was cut, batched or placed: only the order of sums may differ (in
+    bfloat16 a last bit of a sum can move a rounded input of the next product by one step, hence the looser bound)."""
+    e = row_err(got, want).flatten()
+    tol = 2e-5 if dtype == "float32" else 2e-2
+    return float(e.median()) < tol and float((e < 5 * tol).double().mean()) >= 0.9
+
+
+def whole_prompt(model, name, toks, dtype, slot=0, layers_too=False):
+    """The model's logits for the whole prompt in one step, checked against the oracle (bfloat16: under the model's own expert choices)."""
+    dev, n = model.device, len(toks)
+    model.kv.reserve(slot, n)
+    rec = {}
+    got = model.forward(torch.tensor(toks, dtype=torch.int64, device=dev), torch.arange(n, dtype=torch.int32, device=dev),
+                        torch.full((n,), slot, dtype=torch.int32, device=dev), record=rec, tokens_per_seq=[n]).cpu().clone()
+    model.kv.free(slot)
+    routes = {int(k[1:].split(".")[0]): v.cpu() for k, v in rec.items() if k.endswith(".route")}
+    layers, free = [], {}
+    if dtype == "bfloat16":
+        R.forward(config_of(name), make_weights(name), toks, chosen=free)
+        want = R.forward(config_of(name), make_weights(name), toks, layers, routes=routes)
+    else:
+        want = R.forward(config_of(name), make_weights(name), toks, layers, chosen=free)
+    for l, idx in routes.items():
+        if dtype == "bfloat16":
+            same = (idx.long().sort(-1).values == free[l].sort(-1).values).all(-1).double().mean()
+            assert float(same) > 0.8, f"layer {l}: the experts chosen differ from the oracle's for too many tokens"
+        else:
+            assert torch.equal(idx.long(), free[l]), f"layer {l}: experts chosen"
+    if layers_too:
+        for i, x in enumerate(layers):
+            assert agrees(rec[f"l{i}.x"], x, dtype), f"residual after layer {i}"
+    assert agrees(got, want, dtype)
+    return got
+
+
+def close(got, want, tol=2e-5):
+    got, want = torch.as_tensor(got, dtype=torch.float64).cpu(), torch.as_tensor(want, dtype=torch.float64).cpu()
+    return float((got - want).abs().max() / want.abs().max().clamp_min(1e-9)) <= tol
+
+
+def make_model(name, dtype, dev, max_tokens=512, max_seqs=4, seed=0, block=16):
+    from vllm_i64_amd.config import ZabutarConfig
+    from vllm_i64_amd.zabutar import ZabutarModel
+    return ZabutarModel(ZabutarConfig.from_dict(config_of(name)), make_weights(name, seed), device=dev, dtype=dtype, max_seqs=max_seqs,
+                        num_kv_blocks=(max_tokens + block - 1) // block, kv_block=block)
+
+
+def oracle_logits(name, toks, seed=0, layers=None):
+    return R.forward(config_of(name), make_weights(name, seed), toks, layers)
+
+
+def replay(engine, requests, schedule):
+    """schedule: steps of [(id, count)]; every position's logits are asked for.  Returns id -> [T, V] (CPU)."""
+    at = {i: 0 for i in requests}
+    got = {i: [] for i in requests}
+    for step in schedule:
+        entries, end = [], []
+        for i, count in step:
+            lo, hi = at[i], at[i] + count
+            entries.append((i, requests[i][lo:hi], list(range(count))))
+            at[i] = hi
+            if hi == len(requests[i]):
+                end.append(i)
+        lg = engine.step(entries, end=end).cpu()
+        row = 0
+        for i, count in step:
+            got[i].append(lg[row:row + count].clone())
+            row += count
+    return {i: torch.cat(v) for i, v in got.items() if v}
+
+
+class Rows:
+    """Rows of a step for op-level calls: sequences of (slot, first position, count) laid out one after the other."""
+
+    def __init__(self, dev, runs):
+        self.slots = torch.tensor([s for s, p, c in runs for _ in range(c)], dtype=torch.int32, device=dev)
+        self.pos = torch.tensor([p + j for s, p, c in runs for j in range(c)], dtype=torch.int32, device=dev)
+        st = [0]
+        for s, p, c in runs:
+            st.append(st[-1] + c)
+        self.seg = torch.tensor(st, dtype=torch.int32, device=dev)
+        self.nseg, self.n = len(runs), st[-1]
+
+
+def cuts_of(T, sizes):
+    out, at, i = [], 0, 0
+    while at < T:
+        c = min(sizes[i % len(sizes)], T - at)
+        out.append((at, c))
+        at += c
+        i += 1
+    return out
+
+
+# =================================================== mechanisms alone =============================================================
+@pytest.mark.parametrize("epi", ["xielu", "silu_mul"])
+@pytest.mark.parametrize("M", [1, 5, 40, 150])
+@pytest.mark.parametrize("exact", [False, True])
+def test_linear_activation_epilogues(dev, epi, M, exact):
+    from vllm_i64_amd import ops_dense as D
+    g = torch.Generator().manual_seed(M)
+    K, N = 72, 52
+    a = torch.randn(M, K, generator=g)
+    if not exact:
+        a = a.to(torch.bfloat16).float()
+    out = torch.empty(M, N, device=dev)
+    if epi == "xielu":
+        w = (torch.randn(N, K, generator=g) * K ** -0.5).to(torch.bfloat16)
+        b = torch.randn(N, generator=g)
+        pq = torch.tensor([0.3, -0.7], dtype=torch.float64)
+        D.linear(a.to(dev), w.to(dev), out, exact=exact, bias=b.to(dev), epilogue=D.EPI_XIELU, act_a=float(R.softplus(pq[0])), act_b=0.5 + float(R.softplus(pq[1])))
+        want = R.xielu(a.double() @ w.double().T + b.double(), pq)
+        assert float((want > 0).double().mean()) > 0.2 and float((want < 0).double().mean()) > 0.2      # both branches are there
+    else:
+        w = (torch.randn(2 * N, K, generator=g) * K ** -0.5).to(torch.bfloat16)
+        D.linear(a.to(dev), w.to(dev), out, exact=exact, epilogue=D.EPI_SILU_MUL)
+        want = R.silu(a.double() @ w[:N].double().T) * (a.double() @ w[N:].double().T)
+    assert close(out, want, 1e-5)
+
+
+@pytest.mark.parametrize("exact", [False, True])
+@pytest.mark.parametrize("counts", [[3, 0, 70, 1], [0, 0, 5], [130], [64, 64, 1, 0, 0, 9]])
+def test_linear_over_groups_of_rows_counted_on_the_device(dev, exact, counts):
+    """Every group multiplies its own rows (gathered through a row list) by its own weight; empty groups, groups longer than a tile."""
+    from vllm_i64_amd import ops_dense as D
+    g = torch.Generator().manual_seed(sum(counts))
+    K, N, G, total = 40, 24, len(counts), sum(counts)
+    src = torch.randn(total + 7, K, generator=g).to(torch.bfloat16).float()
+    rows = torch.randperm(total + 7, generator=g)[:total].to(torch.int32)
+    w = (torch.randn(G, 2 * N, K, generator=g) * K ** -0.5).to(torch.bfloat16)
+    off = torch.tensor([0] + list(torch.tensor(counts).cumsum(0)), dtype=torch.int32)
+    out = torch.full((total, N), 7.0, device=dev)
+    D.linear(src.to(dev), w.to(dev), out, m=max(counts), a_rows=rows.to(dev), batch=G, w_batch=2 * N * K, exact=exact, epilogue=D.EPI_SILU_MUL, group_off=off.to(dev))
+    want = torch.zeros(total, N, dtype=torch.float64)
+    for b in range(G):
+        x = src[rows[off[b]:off[b + 1]].long()].double()
+        want[off[b]:off[b + 1]] = R.silu(x @ w[b, :N].double().T) * (x @ w[b, N:].double().T)
+    assert close(out, want, 1e-5)
+    w2 = (torch.randn(G, N, K, generator=g) * K ** -0.5).to(torch.bfloat16)
+    out2 = torch.empty(total, N, device=dev)
+    D.linear(src[:total].to(dev).contiguous(), w2.to(dev), out2, m=max(counts), batch=G, w_batch=N * K, exact=exact, group_off=off.to(dev))
+    want2 = torch.cat([src[off[b]:off[b + 1]].double() @ w2[b].double().T for b in range(G)])
+    assert close(out2, want2, 1e-5)
+
+
+def test_embedding_adds_the_row_of_the_position(dev):
+    from vllm_i64_amd import ops_dense as D
+    g = torch.Generator().manual_seed(2)
+    V, W, PMAX = 19, 24, 50
+    table, pos = torch.randn(V, W, generator=g).to(torch.bfloat16), torch.randn(PMAX, W, generator=g).to(torch.bfloat16)
+    r = Rows(dev, [(1, 7, 5), (0, 0, 3), (2, 49, 1)])
+    ids = torch.randint(0, V, (r.n,), generator=g)
+    out = torch.empty(1, r.n, W, device=dev)
+    D.embed_bigram(ids.to(dev), r.pos, r.slots, table.to(dev), out, pos_table=pos.to(dev))
+    want = table[ids].double() + pos[r.pos.cpu().long()].double()
+    assert close(out[0], want, 1e-6)
+
+
+@pytest.mark.parametrize("W", [24, 300])
+def test_residual_adds_the_normed_result_and_norms_for_the_next_sublayer(dev, W):
+    from vllm_i64_amd import ops_dense as D
+    g = torch.Generator().manual_seed(W)
+    n, eps = 7, 1e-5
+    x, y = torch.randn(1, n, W, generator=g), torch.randn(n, W, generator=g) * 3
+    wb, wn = torch.rand(W, generator=g) - 0.5, torch.rand(W, generator=g) - 0.5
+    xs, h = x.to(dev).clone(), torch.empty(n, W, device=dev)
+    D.streams_step(xs, y=y.to(dev), yn_w=(1.0 + wb).to(dev), y_eps=eps, out_w=torch.ones(1, device=dev), norm_w=(1.0 + wn).to(dev), eps=eps, h=h)
+    want_x = x[0].double() + R.offset_norm(y.double(), wb.double(), eps)
+    assert close(xs[0], want_x, 1e-6) and close(h, R.offset_norm(want_x, wn.double(), eps), 1e-5)
+
+
+@pytest.mark.parametrize("taps", [1, 2, 4, 5])
+@pytest.mark.parametrize("cut_sizes", [[40], [1], [2, 5, 1, 3], [600]])
+def test_input_convolution_under_cuts(dev, taps, cut_sizes):
+    """Three sequences in slots whose carried inputs are stale; the cuts fall inside the convolution's reach; 600 rows take the walking kernel."""
+    from vllm_i64_amd import ops_dense as D
+    g = torch.Generator().manual_seed(taps)
+    W = 70
+    lens = {2: 37, 0: 9, 1: 640 if cut_sizes == [600] else 23}
+    w = torch.randn(W, taps, generator=g) * 0.5
+    h = {s: torch.randn(T, W, generator=g) for s, T in lens.items()}
+    want = {s: R.input_convolution(w.double(), h[s].double()) for s in lens}
+    state = torch.full((3, max(taps - 1, 1), W), 9.0, device=dev)[:, : taps - 1] if taps > 1 else None
+    state = state.contiguous() if state is not None else None
+    cuts = {s: cuts_of(T, cut_sizes) for s, T in lens.items()}
+    got = {s: [] for s in lens}
+    for k in range(max(len(c) for c in cuts.values())):
+        runs = [(s, *cuts[s][k]) for s in lens if k < len(cuts[s])]
+        r = Rows(dev, runs)
+        x = torch.cat([h[s][p:p + c] for s, p, c in runs]).to(dev).contiguous()
+        out = torch.empty(r.n, W, device=dev)
+        D.causal_conv(x, off=0, channels=W, w=w.to(dev), bias=None, positions=r.pos, slot_ids=r.slots, state=state, out=out, n=r.n, added=True)
+        row = 0
+        for s, p, c in runs:
+            got[s].append(out[row:row + c].cpu())
+            row += c
+    for s in lens:
+        assert close(torch.cat(got[s]), want[s], 1e-5), s
+
+
+def _hgrn2_weights(H, d, dv, X, g, lower_hi=0.97):
+    return {"q": torch.randn(H * d, X, generator=g) * X ** -0.5, "f": torch.randn(H * d, X, generator=g) * X ** -0.5, "f.b": torch.randn(H * d, generator=g),
+            "lower": torch.rand(H * d, generator=g) * lower_hi, "v": torch.randn(H * dv, X, generator=g) * X ** -0.5, "norm": torch.rand(dv, generator=g) + 0.5,
+            "o": torch.eye(H * dv)}
+
+
+def _hgrn2_run(dev, w, H, d, dv, h, lens_cuts, eps, state):
+    """h: slot -> [T, X]; lens_cuts: slot -> cuts.  Projections on the CPU, everything behind them through the kernels."""
+    from vllm_i64_amd import ops_dense as D
+    nk, nv = H * d, H * dv
+    got = {s: [] for s in h}
+    for k in range(max(len(c) for c in lens_cuts.values())):
+        runs = [(s, *lens_cuts[s][k]) for s in h if k < len(lens_cuts[s])]
+        r = Rows(dev, runs)
+        x = torch.cat([h[s][p:p + c] for s, p, c in runs]).double()
+        P = torch.cat([x @ w["q"].double().T, x @ w["f"].double().T + w["f.b"].double(), x @ w["v"].double().T], 1).float().to(dev).contiguous()
+        cols = dict(q_off=0, f_off=nk, v_off=2 * nk, heads=H, dim=d, vdim=dv, n=r.n)
+        D.gla_gates(P, lower=w["lower"].to(dev), q_act=True, **cols)
+        O, G = torch.empty(r.n, nv, device=dev), torch.empty(r.n, nv, device=dev)
+        D.gla_scan(P, seg_start=r.seg, nseg=r.nseg, positions=r.pos, slot_ids=r.slots, state=state, out=O, **cols)
+        D.gate_norm(O, w["norm"].repeat(H).to(dev), G, groups=H, eps=eps, n=r.n)
+        row = 0
+        for s, p, c in runs:
+            got[s].append(G[row:row + c].cpu())
+            row += c
+    return {s: torch.cat(v) for s, v in got.items()}
+
+
+@pytest.mark.parametrize("H,d,dv", [(3, 40, 24), (2, 16, 64), (1, 130, 8), (5, 8, 33), (2, 64, 20)])
+@pytest.mark.parametrize("cut_sizes", [[200], [1], [2, 5, 1, 3, 90], [7, 2]])
+def test_hgrn2_mechanism_under_cuts(dev, H, d, dv, cut_sizes):
+    g = torch.Generator().manual_seed(H * d + dv)
+    X, eps = 12, 1e-5
+    lens = {1: 150 if cut_sizes != [1] else 40, 3: 11, 0: 64 if cut_sizes != [1] else 20}
+    w = _hgrn2_weights(H, d, dv, X, g)
+    h = {s: torch.randn(T, X, generator=g) for s, T in lens.items()}
+    m = {"heads": H, "dim": d, "vdim": dv}
+    want = {s: R.hgrn2({k: v.double() for k, v in w.items()}, "", m, eps, h[s].double()) for s in lens}
+    state = torch.full((4, H, dv, d), 5.0, device=dev)       # stale: a sequence's first row must not read it
+    got = _hgrn2_run(dev, w, H, d, dv, h, {s: cuts_of(T, cut_sizes) for s, T in lens.items()}, eps, state)
+    for s in lens:
+        assert close(got[s], want[s], 3e-5), s
+
+
+def test_hgrn2_keeps_what_the_gate_keeps_over_hundreds_of_tokens(dev):
+    """Gates bounded below by nearly one on half the channels: the first token's value is still most of the state after 500 tokens, as a
+    prompt and token by token; a state lost at any cut would show as an output without it."""
+    g = torch.Generator().manual_seed(9)
+    H, d, dv, X, eps, T = 2, 12, 10, 6, 1e-6, 500
+    w = _hgrn2_weights(H, d, dv, X, g)
+    w["lower"] = torch.cat([torch.full((d // 2,), 0.998), torch.zeros(d - d // 2)]).repeat(H)
+    w["f.b"] = torch.full((H * d,), 3.0)
+    h = torch.randn(T, X, generator=g) * 0.05
+    h[0] = torch.randn(X, generator=g) * 40.0
+    m = {"heads": H, "dim": d, "vdim": dv}
+    wd = {k: v.double() for k, v in w.items()}
+    want = R.hgrn2(wd, "", m, eps, h.double())
+    h2 = h.clone()
+    h2[0] = 0.0
+    assert row_err(R.hgrn2(wd, "", m, eps, h2.double())[-1:], want[-1:]) > 0.3       # the last output rests on the first token
+    for cuts in ([(0, T)], [(0, T - 40)] + [(t, 1) for t in range(T - 40, T)], cuts_of(T, [64, 2, 100])):
+        state = torch.zeros(2, H, dv, d, device=dev)
+        got = _hgrn2_run(dev, w, H, d, dv, {1: h}, {1: cuts}, eps, state)[1]
+        assert close(got, want, 2e-3), cuts[:3]      # (one minus a gate near one has few digits left in 32 bits; a lost state is off by 30 %)
+
+
+# ---- attention ----------------------------------------------------------------------------------------------------------------------
+class KvPages:
+    """A hand-made paged cache of [values | keys] rows for sequences whose pages are scattered and in no order."""
+
+    def __init__(self, dev, lens, width, block, dtype, seed=0):
+        need = {s: (T + block - 1) // block for s, T in lens.items()}
+        nb = sum(need.values())
+        self.rows = torch.zeros(2 * nb + 3, block, width, dtype=dtype, device=dev)
+        perm = torch.randperm(2 * nb + 3, generator=torch.Generator().manual_seed(seed + nb)).tolist()
+        bt = torch.full((max(lens) + 1, max(need.values())), -1, dtype=torch.int32)
+        for s, k in need.items():
+            for b in range(k):
+                bt[s, b] = perm.pop()
+        self.bt = bt.to(dev)
+
+
+def _attn_weights(H, G, d, dv, X, rel_rows, g, rel_std=2.0):
+    return {"q": torch.randn(H * d, X, generator=g) * X ** -0.5, "k": torch.randn(G * d, X, generator=g) * X ** -0.5, "v": torch.randn(G * dv, X, generator=g) * X ** -0.5,
+            "rel": torch.randn(rel_rows, H, generator=g) * rel_std, "o": torch.eye(H * dv)}
+
+
+def _attn_run(dev, w, m, h, lens_cuts, block, dtype, form, splits=1, round_inputs=False):
+    """h: slot -> [T, X]; one launch per step over every sequence's portion.  form: 'row' (one wave per row and head) or 'mfma'."""
+    from vllm_i64_amd import ops_dense as D
+    from vllm_i64_amd.dogalorn import distance_bias_table
+    H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+    gs = d + dv
+    pages = KvPages(dev, {s: x.shape[0] for s, x in h.items()}, G * gs, block, dtype)
+    bias = distance_bias_table(w["rel"].float(), float(m["bias_max"])).to(dev)
+    got = {s: [] for s in h}
+    for k in range(max(len(c) for c in lens_cuts.values())):
+        runs = [(s, *lens_cuts[s][k]) for s in h if k < len(lens_cuts[s])]
+        r = Rows(dev, runs)
+        x = torch.cat([h[s][p:p + c] for s, p, c in runs]).double()
+        P = torch.cat([x @ w["q"].double().T, x @ w["k"].double().T, x @ w["v"].double().T], 1).float()
+        if round_inputs:
+            P = P.to(torch.bfloat16).float()
+        P = P.to(dev).contiguous()
+        Q, O = torch.empty(r.n, H * gs, device=dev), torch.empty(r.n, H * dv, device=dev)
+        D.kv_prep(P, q_off=0, k_off=H * d, v_off=(H + G) * d, heads=H, kv_heads=G, dim=d, vdim=dv, scale=m["scale"], positions=r.pos, slot_ids=r.slots,
+                  block_table=pages.bt, cache=pages.rows, q=Q, n=r.n)
+        single = all(c == 1 for _, _, c in runs)
+        mode = 1 if form == "row" else (2 if single else 3)
+        D.kattn(Q, pages.rows, None, pages.bt, r.slots, r.pos, chunk=0, bias=bias, sink=False, heads=H, kv_heads=G, dim=d, vdim=dv, out=O, n=r.n, mode=mode,
+                splits=splits if (single and form == "mfma") else 1)
+        row = 0
+        for s, p, c in runs:
+            got[s].append(O[row:row + c].cpu())
+            row += c
+    return {s: torch.cat(v) for s, v in got.items()}
+
+
+def _attn_oracle(w, m, h):
+    wd = {k: v.double() for k, v in w.items()}
+    k, v = R.keys_and_values(wd, "", h.double())
+    return R.biased_attention(wd, "", m, h.double(), k, v)
+
+
+@pytest.mark.parametrize("H,G,d,dv", [(3, 3, 16, 16), (6, 2, 10, 14), (4, 1, 24, 40), (2, 2, 130, 7)])
+@pytest.mark.parametrize("block,cut_sizes", [(16, [300]), (4, [1]), (8, [2, 11, 1, 64]), (16, [33, 2])])
+def test_attention_random_rows_in_32_bits(dev, H, G, d, dv, block, cut_sizes):
+    """Distances run past bias_max and past every bucket's edge with a table of large entries: a bucket that is one off shows."""
+    g = torch.Generator().manual_seed(H * d + dv + block)
+    X = 9
+    m = {"heads": H, "kv_heads": G, "dim": d, "vdim": dv, "scale": 0.37, "bias_max": 57}
+    w = _attn_weights(H, G, d, dv, X, 11, g)
+    lens = {2: 140 if cut_sizes != [1] else 70, 0: 21}
+    h = {s: torch.randn(T, X, generator=g) for s, T in lens.items()}
+    got = _attn_run(dev, w, m, h, {s: cuts_of(T, cut_sizes) for s, T in lens.items()}, block, torch.float32, "row")
+    for s in lens:
+        assert close(got[s], _attn_oracle(w, m, h[s]), 3e-5), s
+
+
+@pytest.mark.parametrize("H,G,d,dv", [(3, 3, 16, 16), (8, 2, 48, 32), (34, 2, 32, 16), (2, 1, 64, 256), (4, 2, 40, 64), (2, 2, 8, 48)])
+@pytest.mark.parametrize("block,cut_sizes", [(16, [200]), (4, [1]), (16, [2, 11, 1, 40])])
+def test_attention_matrix_core_form(dev, H, G, d, dv, block, cut_sizes):
+    """bf16 cache and bf16-representable projections: the cache holds them exactly, what is left is the two-term split of query and weights."""
+    g = torch.Generator().manual_seed(H + d + dv)
+    X = 9
+    m = {"heads": H, "kv_heads": G, "dim": d, "vdim": dv, "scale": 0.3, "bias_max": 30}
+    w = _attn_weights(H, G, d, dv, X, 10, g)
+    T = 90 if cut_sizes != [1] else 50
+    # the projections are the inputs: identity weights over a bf16-representable input of the three parts' total width
+    Xw = (H + G) * d + G * dv
+    w["q"], w["k"], w["v"] = torch.eye(Xw)[: H * d], torch.eye(Xw)[H * d:(H + G) * d], torch.eye(Xw)[(H + G) * d:]
+    h = {1: (torch.randn(T, Xw, generator=g)).to(torch.bfloat16).float()}
+    want = _attn_oracle(w, m, h[1])
+    from vllm_i64_amd import ops_dense as D
+    for single_row_form in ((1, 0) if 1 in cut_sizes else (1,)):
+        D.call_dense("i64h_set_latent_attn_decode_form", single_row_form)
+        try:
+            got = _attn_run(dev, w, m, h, {1: cuts_of(T, cut_sizes)}, block, torch.bfloat16, "mfma", splits=3)
+        finally:
+            D.call_dense("i64h_set_latent_attn_decode_form", 1)
+        assert close(got[1], want, 2e-4), single_row_form
+
+
+def test_attention_batches_of_unequal_rows(dev):
+    """One launch over portions of three sequences whose borders fall inside a tile of 16 rows, and one over single rows of three
+    sequences at different positions, against the oracle on each sequence alone."""
+    g = torch.Generator().manual_seed(11)
+    H, G, d, dv, block = 4, 2, 32, 48, 16
+    m = {"heads": H, "kv_heads": G, "dim": d, "vdim": dv, "scale": 0.25, "bias_max": 20}
+    w = _attn_weights(H, G, d, dv, 8, 6, g)
+    Xw = (H + G) * d + G * dv
+    w["q"], w["k"], w["v"] = torch.eye(Xw)[: H * d], torch.eye(Xw)[H * d:(H + G) * d], torch.eye(Xw)[(H + G) * d:]
+    lens = {0: 38, 1: 6, 2: 61}
+    h = {s: torch.randn(T, Xw, generator=g).to(torch.bfloat16).float() for s, T in lens.items()}
+    want = {s: _attn_oracle(w, m, h[s]) for s in lens}
+    for form, dtype in (("mfma", torch.bfloat16), ("row", torch.float32)):
+        got = _attn_run(dev, w, m, h, {s: [(0, T - 1), (T - 1, 1)] for s, T in lens.items()}, block, dtype, form, splits=2)
+        for s in lens:
+            assert close(got[s], want[s], 2e-4), (form, s)
+
+
+@pytest.mark.parametrize("mode", ["prompt", "decode"])
+@pytest.mark.parametrize("block,T", [(16, 200), (8, 530)])
+def test_attention_one_key_stands_out(dev, mode, block, T):
+    """The last query and ONE key point the same way and are long, every other key is orthogonal to the query: the output is that key's
+    value.  The key is placed at the first position, far back, at page borders and next to the query, with a distance bias that favours
+    another bucket by a margin the aligned score overcomes."""
+    g = torch.Generator().manual_seed(T)
+    H, d, dv = 2, 16, 24
+    m = {"heads": H, "kv_heads": H, "dim": d, "vdim": dv, "scale": 1.0, "bias_max": 64}
+    Xw = 2 * H * d + H * dv
+    w = {"q": torch.eye(Xw)[: H * d], "k": torch.eye(Xw)[H * d:2 * H * d], "v": torch.eye(Xw)[2 * H * d:], "rel": torch.randn(8, H, generator=g), "o": torch.eye(H * dv)}
+    i = T - 1
+    for j in sorted({0, 1, block - 1, block, 3 * block, i - 65, i - 63, i - 1}):
+        h = torch.randn(T, Xw, generator=g)
+        for b in range(H):
+            q = h[i, b * d:(b + 1) * d].clone()
+            kblk = h[:, H * d + b * d: H * d + (b + 1) * d]
+            kblk -= (kblk @ q)[:, None] / (q @ q) * q
+            kblk[j] = q * 4.0
+        want = _attn_oracle(w, m, h)
+        vj = h[j, 2 * H * d:]
+        assert close(want[i], vj, 2e-2), j                  # the oracle itself: the output is the value at j
+        cuts = [(0, T)] if mode == "prompt" else [(0, T - 1), (T - 1, 1)]
+        got = _attn_run(dev, w, m, {1: h}, {1: cuts}, block, torch.float32, "row")[1]
+        assert close(got[i], want[i], 3e-5), j
+        hb = h.to(torch.bfloat16).float()
+        got = _attn_run(dev, w, m, {1: hb}, {1: cuts}, block, torch.bfloat16, "mfma", splits=4)[1]
+        assert close(got[i], _attn_oracle(w, m, hb)[i], 3e-4), (j, "matrix cores")
+
+
+def test_attention_bias_decides_between_equal_scores(dev):
+    """All keys equal: the weights are the softmax of the distance bias alone, so every bucket's edge is in the output.  Values are one-hot
+    by position modulo the value size."""
+    g = torch.Generator().manual_seed(4)
+    H, d, dv, T = 3, 8, 32, 150
+    for rel_rows, far in ((16, 100.0), (7, 29.0), (4, 5.0)):
+        m = {"heads": H, "kv_heads": 1, "dim": d, "vdim": dv, "scale": 0.5, "bias_max": far}
+        Xw = H * d + d + dv
+        w = {"q": torch.eye(Xw)[: H * d], "k": torch.eye(Xw)[H * d: H * d + d], "v": torch.eye(Xw)[H * d + d:], "rel": torch.randn(rel_rows, H, generator=g) * 3, "o": torch.eye(H * dv)}
+        h = torch.zeros(T, Xw)
+        h[:, : H * d] = torch.randn(T, H * d, generator=g)
+        h[:, H * d: H * d + d] = 1.0
+        h[torch.arange(T), H * d + d + torch.arange(T) % dv] = 1.0
+        want = _attn_oracle(w, m, h)
+        got = _attn_run(dev, w, m, {1: h}, {1: [(0, T - 20)] + [(t, 1) for t in range(T - 20, T)]}, 16, torch.float32, "row")[1]
+        assert close(got, want, 3e-5), rel_rows
+        got = _attn_run(dev, w, m, {1: h}, {1: [(0, T - 20)] + [(t, 1) for t in range(T - 20, T)]}, 16, torch.bfloat16, "mfma", splits=2)[1]
+        assert close(got, want, 3e-4), (rel_rows, "matrix cores")
+
+
+# ---- router and experts ----------------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("E,groups,keep,top", [(6, 3, 2, 2), (10, 2, 1, 2), (16, 4, 2, 4), (5, 1, 1, 1), (70, 7, 3, 9), (8, 8, 3, 3), (3, 1, 1, 3)])
+def test_router_choices_and_weights(dev, E, groups, keep, top):
+    from vllm_i64_amd import ops_dense as D
+    g = torch.Generator().manual_seed(E + top)
+    n = 301
+    z = torch.randn(n, E, generator=g) * 2
+    corr = torch.randn(E, generator=g) * 0.4 - (1.0 if E == 10 else 0.0)       # (all choice scores negative for one of the cases)
+    r = {"top": top, "scale": 1.7}
+    if groups > 1:
+        r["groups"] = {"count": groups, "keep": keep}
+    idx, wgt = R.route(z.double(), corr.double(), r)
+    gi, gw = torch.empty(n, top, dtype=torch.int32, device=dev), torch.empty(n, top, device=dev)
+    D.route_topk(z.to(dev), entries=E, correction=corr.to(dev), groups=groups, keep=keep, top=top, scale=1.7, idx=gi, wgt=gw, n=n)
+    assert torch.equal(gi.cpu().long(), idx)          # the same entries in the same order (largest first)
+    assert close(gw, wgt, 1e-5)
+
+
+@pytest.mark.parametrize("name,l", [("odd", 1), ("odd", 3), ("odd", 5), ("plain", 2), ("wide", 0), ("wide", 2)])
+@pytest.mark.parametrize("n", [1, 7, 200])
+def test_mixture_of_experts_alone(dev, name, l, n):
+    model = make_model(name, "float32", dev)
+    cfg, w = config_of(name), {k: v.double() for k, v in make_weights(name).items()}
+    h = torch.randn(n, cfg["width"], generator=torch.Generator().manual_seed(n + l))
+    B = model.buffers(n, 1)
+    B.hc.copy_(h)
+    model._moe_ff(B, model.layers[l], n)
+    want = R.mixture_ff(w, f"l{l}.mlp.", cfg["layers"][l]["mlp"], h.double())
+    assert close(B.y, want, 2e-5)
+
+
+def test_experts_that_get_no_token_and_one_that_gets_all(dev):
+    name, l, n = "odd", 1, 40
+    wts = make_weights(name)
+    wts["l1.mlp.router"] = torch.zeros_like(wts["l1.mlp.router"])
+    wts["l1.mlp.correction"] = torch.tensor([0.0, 0.0, 5.0, 4.0, 0.0, 0.0]).to(torch.bfloat16)     # entries 2 and 3 for every token
+    from vllm_i64_amd.config import ZabutarConfig
+    from vllm_i64_amd.zabutar import ZabutarModel
+    model = ZabutarModel(ZabutarConfig.from_dict(config_of(name)), wts, device=dev, dtype="float32", num_kv_blocks=4)
+    h = torch.randn(n, 40, generator=torch.Generator().manual_seed(3))
+    B = model.buffers(n, 1)
+    B.hc.copy_(h)
+    model._moe_ff(B, model.layers[l], n)
+    assert B.group_off.tolist() == [0, 0, 0, n, 2 * n, 2 * n]
+    want = R.mixture_ff({k: v.double() for k, v in wts.items()}, "l1.mlp.", config_of(name)["layers"][l]["mlp"], h.double())
+    assert close(B.y, want, 2e-5)
+
+
+@pytest.mark.parametrize("n", [3, 100])
+def test_dense_feed_forward_alone(dev, n):
+    model = make_model("odd", "float32", dev)
+    w = {k: v.double() for k, v in make_weights("odd").items()}
+    h = torch.randn(n, 40, generator=torch.Generator().manual_seed(n)) * 2
+    B = model.buffers(n, 1)
+    B.hc.copy_(h)
+    model._dense_ff(B, model.layers[0], n)
+    assert close(B.y, R.dense_ff(w, "l0.mlp.", h.double()), 2e-5)
+
+
+# ===================================================== whole models ===============================================================
+@pytest.mark.parametrize("name", list(SHAPES))
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_whole_prompt_and_residual_after_every_layer(dev, name, dtype):
+    whole_prompt(make_model(name, dtype, dev), name, tokens(name, 140, 1), dtype, slot=2, layers_too=True)
+
+
+@pytest.mark.parametrize("name", list(SHAPES))
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_cuts_batches_and_reuse(dev, name, dtype):
+    """Token by token from the first token; portions of changing size down to two tokens; four live requests of unequal length in a
+    pool that only fits with page reuse, more requests than slots over the run; a request left out of steps.  Every request's whole
+    prompt is checked against the oracle first; the schedules must then give the same logits."""
+    from vllm_i64_amd.engine import Engine
+    model = make_model(name, dtype, dev, max_tokens=4 * 64, max_seqs=4)
+    reqs = {"a": tokens(name, 61, 2), "b": tokens(name, 38, 3), "c": tokens(name, 1, 4), "d": tokens(name, 50, 5), "e": tokens(name, 33, 6), "f": tokens(name, 64, 7)}
+    want = {i: whole_prompt(model, name, t, dtype, slot=3) for i, t in reqs.items()}
+    eng = Engine(model)
+    got = replay(eng, {"b": reqs["b"]}, [[("b", 1)] for _ in range(38)])
+    assert same_to_rounding(got["b"], want["b"], dtype)
+    got = replay(eng, {"a": reqs["a"]}, [[("a", c)] for _, c in cuts_of(61, [2, 17, 1, 3, 16, 2, 5])])
+    assert same_to_rounding(got["a"], want["a"], dtype)
+    sched = [[("a", 30), ("b", 2)], [("a", 1), ("b", 20), ("c", 1), ("d", 7)], [("b", 1), ("d", 2), ("e", 16)], [("a", 28), ("b", 1), ("d", 1), ("e", 1)],
+             [("a", 2), ("b", 14), ("d", 40), ("e", 2)], [("e", 14), ("f", 33)], [("f", 1)], [("f", 30)]]
+    got = replay(eng, reqs, sched)
+    for i in reqs:
+        assert same_to_rounding(got[i], want[i], dtype), i
+    assert model.kv.free_blocks == model.kv.num_blocks and not eng.seqs
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_prefill_equals_token_by_token_to_rounding(dev, dtype):
+    """The same sequence whole, token by token and in portions: the logits agree far more closely than either does with the oracle in
+    bfloat16 (nothing but the order of sums may differ)."""
+    from vllm_i64_amd.engine import Engine
+    name = "wide"
+    toks = tokens(name, 90, 12)
+    eng = Engine(make_model(name, dtype, dev, max_tokens=3 * 96, max_seqs=3))
+    whole = replay(eng, {"x": toks}, [[("x", 90)]])["x"]
+    single = replay(eng, {"y": toks}, [[("y", 1)] for _ in range(90)])["y"]
+    parts = replay(eng, {"z": toks}, [[("z", c)] for _, c in cuts_of(90, [2, 31, 1, 16])])["z"]
+    assert same_to_rounding(single, whole, dtype) and same_to_rounding(parts, whole, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_past_the_bias_table_and_pages(dev, dtype):
+    from vllm_i64_amd.engine import Engine
+    name = "odd"
+    toks = tokens(name, 150, 8)
+    model = make_model(name, dtype, dev, max_tokens=160, max_seqs=1)
+    want = whole_prompt(model, name, toks, dtype)
+    got = replay(Engine(model), {"x": toks}, [[("x", 9)]] + [[("x", 1)] for _ in range(141)])
+    assert same_to_rounding(got["x"], want, dtype)
+
+
+def test_positions_end_with_the_table(dev):
+    from vllm_i64_amd.engine import Engine
+    eng = Engine(make_model("plain", "float32", dev, max_tokens=512, max_seqs=1))
+    eng.step([("x", tokens("plain", 256, 1), [255])])
+    with pytest.raises(RuntimeError):
+        eng.step([("x", [1], [0])])
+
+
+@pytest.mark.parametrize("name", ["odd", "plain"])
+def test_greedy_generation_through_the_engine(dev, name):
+    """More prompts than slots; the engine's own scheduler, batching and sampling; against the oracle's greedy continuation."""
+    from vllm_i64_amd.engine import Engine, SamplingParams
+    model = make_model(name, "float32", dev, max_tokens=3 * 64, max_seqs=2)
+    prompts = [tokens(name, n, 20 + n) for n in (5, 19, 1, 12)]
+    new = 6
+    want = []
+    for p in prompts:
+        t = list(p)
+        for _ in range(new):
+            t.append(int(oracle_logits(name, t)[-1].argmax()))
+        want.append(t[len(p):])
+    eng = Engine(model, max_batch_tokens=16)
+    assert eng.generate(prompts, SamplingParams(max_new_tokens=new)) == want
+
+
+def test_graph_decoder_steps_match_the_oracle(dev):
+    """The batch decoder (a captured HIP graph replayed per step) from the first token on: recurrent state, carried convolution inputs,
+    expert routing and the key / value pages advance inside the graph."""
+    from vllm_i64_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("the batch decoder takes its argmax from the first library, which is not built")
+    from vllm_i64_amd.model import GreedyDecoder
+    name = "odd"
+    model = make_model(name, "float32", dev, max_tokens=256, max_seqs=3)
+    prompts = [tokens(name, n, 40 + n) for n in (4, 11, 7)]
+    dec = GreedyDecoder(model, 3, use_graph=True)
+    dec.prefill([torch.tensor(p) for p in prompts], reserve_extra=8)
+    seqs = [list(p) + [int(t)] for p, t in zip(prompts, dec.tokens.tolist())]
+    for _ in range(5):
+        dec.step()
+        torch.cuda.synchronize()
+        for s, t in zip(seqs, dec.tokens.tolist()):
+            s.append(int(t))
+    for p, s in zip(prompts, seqs):
+        t = list(p)
+        for _ in range(6):
+            t.append(int(oracle_logits(name, t)[-1].argmax()))
+        assert s == t
+
+
+def test_trace_command_on_a_checkpoint_folder(dev, tmp_path):
+    from safetensors.torch import save_file
+    name = "plain"
+    ck = tmp_path / "ck"
+    ck.mkdir()
+    (ck / "config.json").write_text(json.dumps(config_of(name)))
+    save_file(make_weights(name), str(ck / "model.safetensors"))
+    toks = tokens(name, 21, 9)
+    steps = [{"step": 0, "entries": [{"id": "q", "tokens": toks[:10], "want": [0, 9]}], "end": []},
+             {"step": 1, "entries": [{"id": "q", "tokens": toks[10:12], "want": []}], "end": []},
+             {"step": 2, "entries": [{"id": "q", "tokens": toks[12:], "want": [8]}, {"id": "r", "tokens": toks[:3], "want": [2]}], "end": ["q", "r"]}]
+    out = tmp_path / "out"
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", str(ck), "--dtype", "float32", "--out", str(out), "--max-tokens", "128"],
+                       input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [l for l in r.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2"]
+    import numpy as np
+    want = oracle_logits(name, toks)
+    V = SHAPES[name]["vocab"]
+    a = torch.from_numpy(np.fromfile(out / "0.f32", dtype="<f4").reshape(-1, V))
+    c = torch.from_numpy(np.fromfile(out / "2.f32", dtype="<f4").reshape(-1, V))
+    assert not (out / "1.f32").exists()
+    assert agrees(a, want[[0, 9]], "float32") and agrees(c, torch.stack([want[20], want[2]]), "float32")

@@ -268,12 +268,14 @@ class ZabutarModel:
         D.linear(B.hc, d["up"], act, exact=self.exact, bias=d["up_b"], epilogue=D.EPI_XIELU, act_a=d["act_a"], act_b=d["act_b"])
         D.linear(act, d["down"], B.y, exact=self.exact, bias=d["down_b"])
 
-    def _moe_ff(self, B, d, n) -> None:
+    def _moe_ff(self, B, d, n, record=None, l=0) -> None:
         f, ex, W = d["mlp"], self.exact, self.cfg.width
         E, top = f.experts, f.top
         logits = B.act[: n * f.entries].view(n, f.entries)
         D.linear(B.hc, d["router"], logits, exact=ex)
         D.route_topk(logits, entries=f.entries, correction=d["correction"], groups=f.groups, keep=f.keep, top=top, scale=f.scale, idx=B.idx, wgt=B.wgt, n=n)
+        if record is not None:
+            record[f"l{l}.route"] = B.idx[: n * top].view(n, top).clone()
         D.moe_plan(B.idx, n=n, top=top, experts=E, group_off=B.group_off, pair_token=B.pair_token, pair_row=B.pair_row)
         # the (token, expert) pairs lie grouped by expert: one launch runs every expert over its own rows, the counts stay on the device
         act = B.act[: n * top * f.ff].view(n * top, f.ff)
@@ -293,7 +295,7 @@ class ZabutarModel:
         """token_ids int64 [N]; positions / slot_ids int32 [N], rows in sequence order (the rows of a sequence consecutive, positions
         consecutive, continuing what the sequence's slot and pages hold; position 0 starts a sequence afresh); logit_rows int32 [M]
         selects the rows whose logits are wanted (None = all).  Returns fp32 logits [M, V].  record: dict filled with the residual after
-        every layer ("l<i>.x").  kv: a HybridCache other than the runner's own.  tokens_per_seq (rows per sequence, in order) or
+        every layer ("l<i>.x") and every mixture layer's chosen entries ("l<i>.route", int32 [N, top]).  kv: a HybridCache other than the runner's own.  tokens_per_seq (rows per sequence, in order) or
         rows_are_slots (every row a sequence of its own) say how the rows are grouped; without them the slot ids are read back.
         ctx_len and max_ctx_hint belong to the shared step interface."""
         cfg = self.cfg
@@ -317,8 +319,10 @@ class ZabutarModel:
             d = self.layers[l]
             D.causal_conv(B.h, off=0, channels=cfg.width, w=d[f"canon{q}"], bias=None, positions=positions, slot_ids=slot_ids,
                           state=kvc.state[l].get(f"canon{q}"), out=B.hc, n=n, added=True)
-            if q == 2:
-                (self._dense_ff if d["mlp"].kind == "dense" else self._moe_ff)(B, d, n)
+            if q == 2 and d["mlp"].kind == "dense":
+                self._dense_ff(B, d, n)
+            elif q == 2:
+                self._moe_ff(B, d, n, record, l)
             elif d["type"] == "hgrn2":
                 self._hgrn2(B, d, l, n, positions, slot_ids, kvc, seg, nseg)
             else:
