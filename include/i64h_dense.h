@@ -162,6 +162,8 @@ typedef struct {
     const float* bias;   /* fp32 [bias_rows, heads]: bias[min(p - j, bias_rows - 1), h] is added to the score */
     int32_t bias_rows;
     int32_t sink;        /* one more score of zero, without a value, in the softmax's denominator */
+    int32_t key_off;     /* the first key_off columns of a cached row part carry values only: the caller's query is zero there, and the score
+                            products over 32-column steps that lie wholly inside them are left out */
 } i64h_latent_attn_args;
 int i64h_set_latent_attn_decode_form(int32_t on); /* tuning / test knob: 1 (default) = mode 2 launches run the kernel that requests a tile's fragments a tile ahead; 0 = the general matrix-core kernel; same results up to summation order */
 int64_t i64h_latent_attn_workspace_floats(int64_t n, int32_t heads, int32_t kv_rank, int32_t splits);

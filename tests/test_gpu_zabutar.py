@@ -287,6 +287,24 @@ def test_hgrn2_mechanism_under_cuts(dev, H, d, dv, cut_sizes):
         assert close(got[s], want[s], 3e-5), s
 
 
+def test_recurrence_with_keys_of_its_own(dev):
+    """The scan's other form (keys read from the projection rows instead of one minus the gate) with exactly those keys written out."""
+    from vllm_i64_amd import ops_dense as D
+    g = torch.Generator().manual_seed(21)
+    for H, d, dv, runs in ((3, 20, 24, [(0, 0, 70), (2, 0, 9)]), (2, 64, 48, [(1, 0, 33)])):
+        nk, nv = H * d, H * dv
+        r = Rows(dev, runs)
+        P = torch.rand(r.n, 3 * nk + nv, generator=g).to(dev)
+        P[:, 2 * nk:3 * nk] = 1.0 - P[:, nk:2 * nk]
+        outs = []
+        for k_off in (-1, 2 * nk):
+            state, O = torch.zeros(3, H, dv, d, device=dev), torch.empty(r.n, nv, device=dev)
+            D.gla_scan(P, q_off=0, f_off=nk, v_off=3 * nk, heads=H, dim=d, vdim=dv, seg_start=r.seg, nseg=r.nseg, positions=r.pos, slot_ids=r.slots, state=state,
+                       out=O, n=r.n, k_off=k_off)
+            outs.append((O.cpu(), state.cpu()))
+        assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+
+
 def test_hgrn2_keeps_what_the_gate_keeps_over_hundreds_of_tokens(dev):
     """Gates bounded below by nearly one on half the channels: the first token's value is still most of the state after 500 tokens, as a
     prompt and token by token; a state lost at any cut would show as an output without it."""

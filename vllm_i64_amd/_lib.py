@@ -258,7 +258,7 @@ class LatentAttn(ctypes.Structure):
     _fields_ = [("Q", _P), ("cache", _P), ("cache_dtype", _I), ("block_table", _P), ("max_blocks_per_seq", _I), ("block_size", _I),
                 ("slot_ids", _P), ("positions", _P), ("window", _I), ("scale", _F), ("out", _P), ("n", _L), ("heads", _I), ("kv_rank", _I),
                 ("rot_dim", _I), ("mode", _I), ("splits", _I), ("workspace", _P), ("row_stride", _I), ("kv_groups", _I), ("chunk", _I), ("kscale", _P),
-                ("bias", _P), ("bias_rows", _I), ("sink", _I)]
+                ("bias", _P), ("bias_rows", _I), ("sink", _I), ("key_off", _I)]
 
 
 class EmbedBigram(ctypes.Structure):

@@ -1,7 +1,8 @@
-"""`bench.py --design morilorn | dogalorn`: prefill and decode throughput of a registered design at layer sizes of real models (random
-weights), beside the package's closest existing model at equal width, depth, feed-forward size and batch (Morilorn: the dense int8
-decoder; Dogalorn: Morilorn, which shares its library, bf16 Linears and 32-bit residual), and the design's kernels one by one
-against their rooflines beside the like kernel of that model.  Prints one JSON line."""
+"""`bench.py --design morilorn | dogalorn | zabutar`: prefill and decode throughput of a registered design at layer sizes of real models
+(random weights), beside the package's closest existing model at equal width, depth, feed-forward size and batch (Morilorn: the dense
+int8 decoder; Dogalorn: Morilorn, which shares its library, bf16 Linears and 32-bit residual; Zabutar: Dogalorn, the other design of
+recurrent layers beside attention with a distance bias), and the design's kernels one by one against their rooflines beside the like
+kernel of that model.  Prints one JSON line."""
 from __future__ import annotations
 
 import json
@@ -337,6 +338,192 @@ def run_dogalorn(args) -> dict:
     return result
 
 
+ZABUTAR_SIZES = {
+    "w1024": dict(width=1024, blocks=4, rec_heads=8, rec_dim=128, rec_vdim=128, heads=16, kv_heads=4, dim=64, vdim=64, ff=4096, experts=8, top=2, expert_ff=1024,
+                  shared_ff=1024),
+    "w2048": dict(width=2048, blocks=2, rec_heads=16, rec_dim=128, rec_vdim=128, heads=32, kv_heads=8, dim=64, vdim=64, ff=8192, experts=8, top=2, expert_ff=2048,
+                  shared_ff=2048),
+}
+
+
+def _zabutar_kernels(sz, rows, batch, ctx, dev):
+    """Single launches at the step's shapes with the share of their roofline (matrix products: bf16 matrix peak over the products the
+    design asks for; recurrences: the larger of bytes / HBM rate and flop / fp32 vector rate; everything else: bytes / HBM rate), beside the
+    like kernel of Dogalorn."""
+    from . import ops_dense as D
+    W, ff, H, G, dm, dv = sz["width"], sz["ff"], sz["heads"], sz["kv_heads"], sz["dim"], sz["vdim"]
+    Hr, dk, dr = sz["rec_heads"], sz["rec_dim"], sz["rec_vdim"]
+    E, top, eff = sz["experts"], sz["top"], sz["expert_ff"]
+    dz = DOGALORN_SIZES["w2048" if W >= 2048 else "w1024"]
+    out = {}
+    g = torch.Generator(device=dev).manual_seed(1)
+    rn = lambda *s: torch.randn(*s, device=dev, generator=g)
+
+    def row(name, t, flops=0.0, bytes_=0.0, peak=BF16_TFLOPS):
+        share = max(flops / t / (peak * 1e12), bytes_ / t / (HBM_GBS * 1e9))
+        out[name] = {"us": round(t * 1e6, 1), "roofline_share": round(share, 3)}
+
+    seq = 512
+    warm_a, warm_w, warm_c = rn(rows, W), (rn(W, W) * 0.02).to(torch.bfloat16), torch.empty(rows, W, device=dev)
+    _time(lambda: D.linear(warm_a, warm_w, warm_c), 20)      # clocks and caches settle before the first timed launch
+    for n, tag in ((rows, "prefill"), (batch, "decode")):
+        nseq = n // seq if tag == "prefill" else n
+        per = seq if tag == "prefill" else 1
+        pos0 = 0 if tag == "prefill" else ctx - 1
+        pos = (torch.arange(per, dtype=torch.int32) + pos0).repeat(nseq).to(dev)
+        slots = torch.arange(nseq, dtype=torch.int32).repeat_interleave(per).to(dev)
+        seg = (torch.arange(nseq + 1, dtype=torch.int32) * per).to(dev)
+        reps = 5 if tag == "prefill" else 20
+        a = rn(n, W)
+        # dense feed-forward: up-projection with bias and activation (the same Linear under both designs, another epilogue)
+        w_up, b_up = (rn(ff, W) * 0.02).to(torch.bfloat16), rn(ff)
+        act = torch.empty(n, ff, device=dev)
+        t = _time(lambda: D.linear(a, w_up, act, bias=b_up, epilogue=D.EPI_XIELU, act_a=0.7, act_b=1.2), reps)
+        row(f"linear_up_bias_xielu_{tag}", t, flops=2.0 * n * ff * W, bytes_=2.0 * ff * W + 4.0 * n * (W + ff))
+        t = _time(lambda: D.linear(a, w_up, act, bias=b_up, epilogue=D.EPI_GELU_ERF), reps)
+        row(f"dogalorn_linear_up_bias_gelu_{tag}", t, flops=2.0 * n * ff * W, bytes_=2.0 * ff * W + 4.0 * n * (W + ff))
+        # mixture of experts: router choice, grouping, the two grouped Linears, the weighted sum (beside the dense gate / up pair of equal work)
+        ent = E + 2
+        logits = rn(n, ent) * 2
+        idx, wgt = torch.empty(n, top, dtype=torch.int32, device=dev), torch.empty(n, top, device=dev)
+        corr = torch.zeros(ent, device=dev)
+        t = _time(lambda: D.route_topk(logits, entries=ent, correction=corr, groups=2, keep=1, top=top, scale=1.0, idx=idx, wgt=wgt, n=n), reps)
+        row(f"route_topk_{tag}", t, bytes_=4.0 * n * (ent + 2 * top))
+        goff, ptok, prow = torch.empty(E + 1, dtype=torch.int32, device=dev), torch.empty(n * top, dtype=torch.int32, device=dev), torch.empty(n * top, dtype=torch.int32, device=dev)
+        t = _time(lambda: D.moe_plan(idx, n=n, top=top, experts=E, group_off=goff, pair_token=ptok, pair_row=prow), reps)
+        row(f"moe_plan_{tag}", t, bytes_=4.0 * n * top * 3)
+        pairs = int(goff[-1])
+        w_gu = (rn(E, 2 * eff, W) * 0.02).to(torch.bfloat16)
+        eact, ey = torch.empty(n * top, eff, device=dev), torch.empty(n * top, W, device=dev)
+        t = _time(lambda: D.linear(a, w_gu, eact, m=n, a_rows=ptok, batch=E, w_batch=2 * eff * W, epilogue=D.EPI_SILU_MUL, group_off=goff), reps)
+        row(f"experts_gate_up_{tag}", t, flops=2.0 * pairs * 2 * eff * W, bytes_=2.0 * E * 2 * eff * W + 4.0 * pairs * (W + eff))
+        w_dn = (rn(E, W, eff) * 0.02).to(torch.bfloat16)
+        t = _time(lambda: D.linear(eact, w_dn, ey, m=n, batch=E, w_batch=W * eff, group_off=goff), reps)
+        row(f"experts_down_{tag}", t, flops=2.0 * pairs * eff * W, bytes_=2.0 * E * eff * W + 4.0 * pairs * (W + eff))
+        w_dgu = (rn(2 * top * eff, W) * 0.02).to(torch.bfloat16)      # a dense pair of the same number of products
+        dact = torch.empty(n, top * eff, device=dev)
+        t = _time(lambda: D.linear(a, w_dgu, dact, epilogue=D.EPI_GELU_MUL), reps)
+        row(f"morilorn_linear_gate_up_{tag}", t, flops=2.0 * n * 2 * top * eff * W, bytes_=2.0 * 2 * top * eff * W + 4.0 * n * (W + top * eff))
+        sh, yo = rn(n, W), torch.empty(n, W, device=dev)
+        t = _time(lambda: D.moe_combine(ey, prow, wgt, a, sh, yo, n=n, top=top, width=W), reps)
+        row(f"moe_combine_{tag}", t, bytes_=4.0 * n * W * (top + 3))
+        # residual: add the normed result, norm for the next sublayer; beside Dogalorn's two-stream step
+        st, y, h = rn(1, n, W), rn(n, W), torch.empty(n, W, device=dev)
+        nb_, nw, one = torch.ones(W, device=dev), torch.ones(W, device=dev), torch.ones(1, device=dev)
+        t = _time(lambda: D.streams_step(st, y=y, yn_w=nb_, y_eps=1e-6, out_w=one, norm_w=nw, eps=1e-6, h=h), reps)
+        row(f"sandwich_residual_{tag}", t, bytes_=4.0 * n * W * 4)
+        S = 2
+        st2 = rn(S, n, W)
+        mix, ow, iw, nw1 = torch.eye(S, device=dev), torch.ones(S, device=dev), torch.full((S,), 0.5, device=dev), torch.ones(1, device=dev)
+        t = _time(lambda: D.streams_step(st2, y=y, mix=mix, out_w=ow, in_w=iw, norm_w=nw1, eps=1e-6, h=h), reps)
+        row(f"dogalorn_streams_step_{tag}", t, bytes_=4.0 * n * W * (2 * S + 2))
+        # the convolution added to every sublayer's input; beside Dogalorn's convolution + silu over the state-space channels
+        cw, cstate, hc = rn(W, 4) * 0.1, torch.zeros(nseq, 3, W, device=dev), torch.empty(n, W, device=dev)
+        t = _time(lambda: D.causal_conv(a, off=0, channels=W, w=cw, bias=None, positions=pos, slot_ids=slots, state=cstate, out=hc, n=n, added=True), reps)
+        row(f"input_conv_{tag}", t, bytes_=4.0 * n * W * 2)
+        ch = dz["ssm_heads"] * dz["ssm_vdim"] + 2 * dz["ssm_state"]
+        Pm, cw2, cb2 = rn(n, ch), rn(ch, 4) * 0.3, rn(ch) * 0.1
+        cstate2, xbc = torch.zeros(nseq, 3, ch, device=dev), torch.empty(n, ch, device=dev)
+        t = _time(lambda: D.causal_conv(Pm, off=0, channels=ch, w=cw2, bias=cb2, positions=pos, slot_ids=slots, state=cstate2, out=xbc, n=n), reps)
+        row(f"dogalorn_causal_conv_{tag}", t, bytes_=4.0 * n * ch * 2)
+        # gated linear recurrence: gates, scan, head norm; beside Dogalorn's state-space scan
+        nk, nv = Hr * dk, Hr * dr
+        P = rn(n, 2 * nk + nv) * 0.5
+        lower = torch.rand(nk, device=dev, generator=g) * 0.9
+        cols = dict(q_off=0, f_off=nk, v_off=2 * nk, heads=Hr, dim=dk, vdim=dr, n=n)
+        t = _time(lambda: D.gla_gates(P, lower=lower, q_act=True, **cols), reps)
+        row(f"gla_gates_{tag}", t, bytes_=4.0 * n * nk * 4)
+        P.uniform_(0.0, 1.0)
+        rstate, ro, rg = torch.zeros(nseq, Hr, dr, dk, device=dev), torch.empty(n, nv, device=dev), torch.empty(n, nv, device=dev)
+        t = _time(lambda: D.gla_scan(P, seg_start=seg, nseg=nseq, positions=pos, slot_ids=slots, state=rstate, out=ro, **cols), reps)
+        row(f"gla_scan_{tag}", t, flops=5.0 * n * Hr * dk * dr, bytes_=4.0 * n * (2 * nk + 2 * nv) + 8.0 * nseq * Hr * dk * dr, peak=F32_TFLOPS)
+        t = _time(lambda: D.gate_norm(ro, torch.ones(nv, device=dev), rg, groups=Hr, eps=1e-6, n=n), reps)
+        row(f"head_norm_{tag}", t, bytes_=4.0 * n * nv * 2)
+        Hs, Pv, N = dz["ssm_heads"], dz["ssm_vdim"], dz["ssm_state"]
+        inner, chs = Hs * Pv, Hs * Pv + 2 * N
+        Ps, xs = rn(n, inner + chs + Hs) * 0.5, rn(n, chs) * 0.5
+        sstate, yv = torch.zeros(nseq, Hs, Pv, N, device=dev), torch.empty(n, inner, device=dev)
+        dtb, al, dkp = torch.full((Hs,), -2.0, device=dev), torch.zeros(Hs, device=dev), torch.ones(Hs, device=dev)
+        t = _time(lambda: D.ssm_scan(xs, Ps, dt_off=inner + chs, lddt=inner + chs + Hs, dt_bias=dtb, a_log=al, d_skip=dkp, heads=Hs, vdim=Pv, state=N, groups=1,
+                                     seg_start=seg, nseg=nseq, positions=pos, slot_ids=slots, ssm_state=sstate, y=yv, n=n), reps)
+        row(f"dogalorn_ssm_scan_{tag}", t, flops=6.0 * n * Hs * N * Pv, bytes_=4.0 * n * (chs + inner) + 8.0 * nseq * Hs * N * Pv, peak=F32_TFLOPS)
+        # attention: a prompt's rows, and one row per sequence at context ctx; beside Dogalorn's attention whose values are the keys
+        plen = seq if tag == "prefill" else ctx
+        nb = (plen + 15) // 16
+        bt = torch.arange(nseq * nb, dtype=torch.int32, device=dev).view(nseq, nb).contiguous()
+        gs = dv + dm
+        kc = (rn(nseq * nb, 16, G * gs) * 0.5).to(torch.bfloat16)
+        Pq = rn(n, H * dm) * 0.3
+        q, oa = torch.empty(n, H * gs, device=dev), torch.empty(n, H * dv, device=dev)
+        t = _time(lambda: D.kv_prep(Pq, q_off=0, k_off=0, v_off=0, heads=H, kv_heads=G, dim=dm, vdim=dv, scale=0.125, positions=pos, slot_ids=slots, block_table=bt,
+                                    cache=None, q=q, n=n, block_size=16), reps)
+        row(f"kv_prep_queries_{tag}", t, bytes_=4.0 * n * H * (dm + gs))
+        bias = torch.zeros(4097, H, device=dev)
+        keys = seq * (seq + 1) / 2 * nseq if tag == "prefill" else float(ctx) * n
+        waves = 3072 if gs <= 64 else (2048 if gs <= 128 else 1024)
+        sp = 1 if tag == "prefill" else max(1, min(waves // max(1, n * G * ((H // G + 15) // 16)), int(keys / n) // 64, 64))
+        t = _time(lambda: D.kattn(q, kc, None, bt, slots, pos, chunk=0, bias=bias, sink=False, heads=H, kv_heads=G, dim=dm, vdim=dv, out=oa, n=n,
+                                  mode=3 if tag == "prefill" else 2, splits=sp), reps)
+        row(f"kv_attention_{tag}", t, flops=2.0 * keys * H * (dm + dv), bytes_=(2.0 * keys * G * gs if tag == "decode" else 0.0) + 4.0 * n * H * (gs + dv))
+        kc2 = (rn(nseq * nb, 16, G * dm) * 0.5).to(torch.bfloat16)
+        ks = torch.rand(nseq * nb, 16, device=dev, generator=g) + 0.5
+        q2, oa2 = rn(n, H * dm) * 0.3, torch.empty(n, H * dm, device=dev)
+        sp2 = 1 if tag == "prefill" else max(1, min((3072 if dm <= 64 else 1024) // max(1, n * G * ((H // G + 15) // 16)), int(keys / n) // 64, 64))
+        t = _time(lambda: D.kattn(q2, kc2, ks, bt, slots, pos, chunk=4096, bias=bias, sink=True, heads=H, kv_heads=G, dim=dm, out=oa2, n=n,
+                                  mode=3 if tag == "prefill" else 2, splits=sp2), reps)
+        row(f"dogalorn_kattn_{tag}", t, flops=4.0 * keys * H * dm, bytes_=(2.0 * keys * G * dm if tag == "decode" else 0.0) + 8.0 * n * H * dm)
+    return out
+
+
+def run_zabutar(args) -> dict:
+    from . import _lib, synth
+    from .dogalorn import DogalornModel
+    from .model import GreedyDecoder
+    from .zabutar import ZabutarModel
+    _lib.load(), _lib.load_dense()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    batch, ctx, rows = args.batch, args.prompt_len, 4096
+    result = {"metric": "prefill / decode tokens/s of the Zabutar design beside Dogalorn at equal sizes", "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+              "warmup": args.warmup, "dtype": "bf16 matrix products, fp32 residual / norms / recurrences / attention math (both designs)", "data": "synthetic",
+              "config": {"batch": batch, "context": ctx, "prefill_step": f"{rows} rows = {rows // 512} prompts of 512 tokens"}, "sizes": {}}
+    for name in (args.design_sizes.split(",") if args.design_sizes else sorted(ZABUTAR_SIZES)):
+        sz = ZABUTAR_SIZES[name]
+        need_tokens = batch * (ctx + args.steps + args.warmup + 64)
+
+        def fill(m):
+            g = torch.Generator(device=dev).manual_seed(5)
+            for t in {id(t): t for t in m.kv.rows if t is not None}.values():
+                t.copy_((0.5 * torch.randn(t.shape, device=dev, generator=g)).to(t.dtype))
+            for t in m.kv.kscale:
+                if t is not None:
+                    t.fill_(2.0)
+            for d in m.kv.state:
+                for t in d.values():
+                    t.copy_(0.1 * torch.randn(t.shape, device=dev, generator=g))
+
+        cfg = synth.zabutar_config(max_positions=max(4096, ctx + args.steps + args.warmup + 64), **sz)
+        model = ZabutarModel(cfg, synth.make_zabutar_weights(cfg), device=dev, dtype="bfloat16", max_seqs=batch, num_kv_blocks=need_tokens // 16)
+        p, d, ms = _steps(model, GreedyDecoder, batch, ctx, rows, 512, args.steps, args.warmup, fill, cfg.vocab, dev)
+        entry = {"zabutar": {"prefill_tokens_per_s": round(p, 1), "decode_tokens_per_s": round(d, 1), "decode_ms_per_step": round(ms, 3), "layers": cfg.num_layers,
+                             "shape": sz}}
+        del model
+        torch.cuda.empty_cache()
+        dz = DOGALORN_SIZES[name]
+        dcfg = synth.dogalorn_config(**dz)
+        dm = DogalornModel(dcfg, synth.make_dogalorn_weights(dcfg), device=dev, dtype="bfloat16", max_seqs=batch, num_kv_blocks=need_tokens // 16)
+        p, d, ms = _steps(dm, GreedyDecoder, batch, ctx, rows, 512, args.steps, args.warmup, fill, dcfg.vocab, dev)
+        entry["dogalorn"] = {"prefill_tokens_per_s": round(p, 1), "decode_tokens_per_s": round(d, 1), "decode_ms_per_step": round(ms, 3), "layers": dcfg.num_layers}
+        del dm
+        torch.cuda.empty_cache()
+        entry["kernels"] = _zabutar_kernels(sz, rows, batch, ctx, dev)
+        result["sizes"][name] = entry
+    first = result["sizes"][sorted(result["sizes"])[0]]["zabutar"]
+    result["value"], result["ms_per_step"] = first["decode_tokens_per_s"], first["decode_ms_per_step"]
+    result["higher_is_better"], result["scaling"], result["vs_baseline"] = True, "weak", None
+    return result
+
+
 def main(args) -> int:
-    print(json.dumps(run_dogalorn(args) if args.design == "dogalorn" else run(args)), flush=True)
+    print(json.dumps({"dogalorn": run_dogalorn, "zabutar": run_zabutar}.get(args.design, run)(args)), flush=True)
     return 0

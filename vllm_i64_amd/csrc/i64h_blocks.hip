@@ -26,11 +26,12 @@ __global__ __launch_bounds__(256) void gla_gates_kernel(const i64h_gla_args p) {
 
 // One workgroup per (head, 16 * CPT value columns, run of rows).  The 16 lanes of a DPP row share CPT neighbouring value columns and hold
 // KPT consecutive key channels of each in registers; a wave has four such rows.  Per token a lane loads its slices of the query, the
-// decay and (where it is not one minus the decay) the key once for its CPT columns - the next token's while this one is computed -,
-// updates its states with fused multiply-adds and the row sums the partial outputs with DPP moves: no LDS and no barrier, the tokens of
-// a run strictly in their order (the same sums in the same order however a prompt is cut).  State layout [slot, head, value column,
-// key channel].
-template <int KPT, int CPT>
+// decay and (where it is not one minus the decay) the key once for its CPT columns, updates its states with fused multiply-adds and
+// the row sums the partial outputs with DPP moves: no LDS and no barrier, the tokens of a run strictly in their order (the same sums in
+// the same order however a prompt is cut).  Loads run GL_TG tokens ahead in two alternating register sets, so that a wave that is alone
+// on its SIMD still has a group of tokens in flight while it computes one.  State layout [slot, head, value column, key channel].
+#define GL_TG 4
+template <int KPT, int CPT, bool HASK>
 __global__ __launch_bounds__(256) void gla_scan_kernel(const i64h_gla_args p, const int ctiles, const int vec) {
     const int N = p.dim, P = p.vdim;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -48,13 +49,28 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(const i64h_gla_args p, co
         const bool cok = cbase + j < P;
         const float* src = gS + (int64_t)(cok ? cbase + j : 0) * N;
 #pragma unroll
-        for (int k = 0; k < KPT; ++k) S[j][k] = (!fresh && cok && n0 + k < N) ? src[k] : 0.0f;
+        for (int k = 0; k < KPT; ++k) S[j][k] = 0.0f;
+        if (!fresh && cok) {
+            if (vec) {
+#pragma unroll
+                for (int k = 0; k < KPT; k += 4)
+                    if (n0 + k < N) {
+                        const float4 v = *(const float4*)(src + k);
+                        S[j][k] = v.x, S[j][k + 1] = v.y, S[j][k + 2] = v.z, S[j][k + 3] = v.w;
+                    }
+            } else {
+#pragma unroll
+                for (int k = 0; k < KPT; ++k)
+                    if (n0 + k < N) S[j][k] = src[k];
+            }
+        }
     }
-    const int qoff = p.q_off + a * N + n0, foff = p.f_off + a * N + n0, koff = p.k_off >= 0 ? p.k_off + a * N + n0 : -1;
+    const int qoff = p.q_off + a * N + n0, foff = p.f_off + a * N + n0, koff = HASK ? p.k_off + a * N + n0 : 0;
     struct Tok {
-        float q[KPT], f[KPT], k[KPT], v[CPT];
+        float q[KPT], f[KPT], k[HASK ? KPT : 1], v[CPT];
     };
     auto fetch = [&](int64_t t, Tok& u) {
+        if (t >= r1) return;
         const float* row = p.P + t * p.ldp;
         if (vec) {      // KPT % 4 == 0 and every slice starts at a multiple of four floats and lies inside the row
 #pragma unroll
@@ -63,11 +79,11 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(const i64h_gla_args p, co
                 if (n0 + k < N) {
                     q = *(const float4*)(row + qoff + k);
                     f = *(const float4*)(row + foff + k);
-                    if (koff >= 0) kk = *(const float4*)(row + koff + k);
+                    if (HASK) kk = *(const float4*)(row + koff + k);
                 }
                 u.q[k] = q.x, u.q[k + 1] = q.y, u.q[k + 2] = q.z, u.q[k + 3] = q.w;
                 u.f[k] = f.x, u.f[k + 1] = f.y, u.f[k + 2] = f.z, u.f[k + 3] = f.w;
-                u.k[k] = kk.x, u.k[k + 1] = kk.y, u.k[k + 2] = kk.z, u.k[k + 3] = kk.w;
+                if (HASK) u.k[k] = kk.x, u.k[k + 1] = kk.y, u.k[k + 2] = kk.z, u.k[k + 3] = kk.w;
             }
         } else {
 #pragma unroll
@@ -75,46 +91,53 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(const i64h_gla_args p, co
                 const bool ok = n0 + k < N;
                 u.q[k] = ok ? row[qoff + k] : 0.0f;
                 u.f[k] = ok ? row[foff + k] : 1.0f;
-                u.k[k] = (ok && koff >= 0) ? row[koff + k] : 0.0f;
+                if (HASK) u.k[k] = ok ? row[koff + k] : 0.0f;
             }
-        }
-        if (koff < 0) {
-#pragma unroll
-            for (int k = 0; k < KPT; ++k) u.k[k] = 1.0f - u.f[k];
         }
 #pragma unroll
         for (int j = 0; j < CPT; ++j) u.v[j] = cbase + j < P ? row[p.v_off + a * P + cbase + j] : 0.0f;
     };
     auto step = [&](int64_t t, const Tok& u) {
+        if (t >= r1) return;
 #pragma unroll
         for (int j = 0; j < CPT; ++j) {
             float part = 0.0f;
 #pragma unroll
             for (int k = 0; k < KPT; ++k) {
-                S[j][k] = fmaf(u.f[k], S[j][k], u.k[k] * u.v[j]);
+                const float kk = HASK ? u.k[k] : 1.0f - u.f[k];
+                S[j][k] = fmaf(u.f[k], S[j][k], kk * u.v[j]);
                 part = fmaf(S[j][k], u.q[k], part);
             }
             part = group_sum(part, 16);
             if (nlane == 0 && cbase + j < P) p.out[t * p.ldo + a * P + cbase + j] = part;
         }
     };
-    Tok u0, u1;
-    fetch(r0, u0);
-    for (int64_t t = r0; t < r1; t += 2) {
-        if (t + 1 < r1) fetch(t + 1, u1);
-        step(t, u0);
-        if (t + 1 < r1) {
-            if (t + 2 < r1) fetch(t + 2, u0);
-            step(t + 1, u1);
-        }
+    Tok A[GL_TG], B[GL_TG];
+#pragma unroll
+    for (int i = 0; i < GL_TG; ++i) fetch(r0 + i, A[i]);
+    for (int64_t t = r0; t < r1; t += 2 * GL_TG) {
+#pragma unroll
+        for (int i = 0; i < GL_TG; ++i) fetch(t + GL_TG + i, B[i]);
+#pragma unroll
+        for (int i = 0; i < GL_TG; ++i) step(t + i, A[i]);
+#pragma unroll
+        for (int i = 0; i < GL_TG; ++i) fetch(t + 2 * GL_TG + i, A[i]);
+#pragma unroll
+        for (int i = 0; i < GL_TG; ++i) step(t + GL_TG + i, B[i]);
     }
 #pragma unroll
     for (int j = 0; j < CPT; ++j) {
         if (cbase + j >= P) continue;
         float* dst = gS + (int64_t)(cbase + j) * N;
+        if (vec) {
 #pragma unroll
-        for (int k = 0; k < KPT; ++k)
-            if (n0 + k < N) dst[k] = S[j][k];
+            for (int k = 0; k < KPT; k += 4)
+                if (n0 + k < N) *(float4*)(dst + k) = make_float4(S[j][k], S[j][k + 1], S[j][k + 2], S[j][k + 3]);
+        } else {
+#pragma unroll
+            for (int k = 0; k < KPT; ++k)
+                if (n0 + k < N) dst[k] = S[j][k];
+        }
     }
 }
 
@@ -279,27 +302,28 @@ int i64h_gla_scan(const i64h_gla_args* dp, void* stream) {
     I64H_CHECK_ARG(d.nseg <= 65535, "gla_scan: %d runs in one launch", d.nseg);
     if (d.nseg <= 0 || d.n == 0) return 0;
     const int kpt = (d.dim + 15) / 16;
-    const int cpt = d.vdim > 16 ? 2 : 1;             // columns per lane: query, decay and key are loaded once for both
+    // columns per lane: query, decay and key are loaded once for both - unless the launch would then leave most of the chip idle
+    const int cpt = (d.vdim > 16 && (int64_t)d.heads * ((d.vdim + 31) / 32) * d.nseg >= 512) ? 2 : 1;
     const int ctiles = (d.vdim + 16 * cpt - 1) / (16 * cpt);
     const dim3 grid((unsigned)(d.heads * ctiles), (unsigned)d.nseg);
+    const bool hask = d.k_off >= 0;
     auto launch = [&](auto kern, int K) {
-        const int vec = K % 4 == 0 && d.dim % 4 == 0 && d.ldp % 4 == 0 && d.q_off % 4 == 0 && d.f_off % 4 == 0 && (d.k_off < 0 || d.k_off % 4 == 0) &&
-                        (uintptr_t)d.P % 16 == 0;
+        const int vec = K % 4 == 0 && d.dim % 4 == 0 && d.ldp % 4 == 0 && d.q_off % 4 == 0 && d.f_off % 4 == 0 && (!hask || d.k_off % 4 == 0) &&
+                        (uintptr_t)d.P % 16 == 0 && (uintptr_t)d.state % 16 == 0;
         hipLaunchKernelGGL(kern, grid, dim3(256), 0, (hipStream_t)stream, d, ctiles, vec);
     };
+#define GLA_PICK(C, HK)                                          \
+    if (kpt <= 1) launch(gla_scan_kernel<1, C, HK>, 1);          \
+    else if (kpt <= 2) launch(gla_scan_kernel<2, C, HK>, 2);     \
+    else if (kpt <= 4) launch(gla_scan_kernel<4, C, HK>, 4);     \
+    else if (kpt <= 8) launch(gla_scan_kernel<8, C, HK>, 8);     \
+    else launch(gla_scan_kernel<16, C, HK>, 16);
     if (cpt == 2) {
-        if (kpt <= 1) launch(gla_scan_kernel<1, 2>, 1);
-        else if (kpt <= 2) launch(gla_scan_kernel<2, 2>, 2);
-        else if (kpt <= 4) launch(gla_scan_kernel<4, 2>, 4);
-        else if (kpt <= 8) launch(gla_scan_kernel<8, 2>, 8);
-        else launch(gla_scan_kernel<16, 2>, 16);
+        if (hask) { GLA_PICK(2, true) } else { GLA_PICK(2, false) }
     } else {
-        if (kpt <= 1) launch(gla_scan_kernel<1, 1>, 1);
-        else if (kpt <= 2) launch(gla_scan_kernel<2, 1>, 2);
-        else if (kpt <= 4) launch(gla_scan_kernel<4, 1>, 4);
-        else if (kpt <= 8) launch(gla_scan_kernel<8, 1>, 8);
-        else launch(gla_scan_kernel<16, 1>, 16);
+        if (hask) { GLA_PICK(1, true) } else { GLA_PICK(1, false) }
     }
+#undef GLA_PICK
     I64H_CHECK_LAUNCH();
     return 0;
 }

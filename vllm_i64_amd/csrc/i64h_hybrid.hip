@@ -691,6 +691,7 @@ int i64h_kattn(const i64h_kattn_args* dp, void* stream) {
         a.heads = d.heads, a.kv_rank = vals, a.rot_dim = gs - vals, a.mode = d.mode == 3 ? 3 : 2, a.splits = d.splits, a.workspace = d.workspace;
         a.row_stride = d.kv_heads * gs, a.kv_groups = d.kv_heads, a.chunk = d.chunk, a.kscale = d.kscale, a.bias = d.bias, a.bias_rows = d.bias_rows;
         a.sink = d.sink;
+        a.key_off = d.vdim > 0 ? d.vdim : 0;
         return i64h_latent_attn(&a, stream);
     }
     const int64_t items = d.n * d.heads;

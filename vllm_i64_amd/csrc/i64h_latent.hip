@@ -283,8 +283,10 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, KD > 4 ? 
                     if (ks * 32 < D) {
                         const int d0 = ks * 32 + kg * 8;
                         const uint4 kf = d0 < D ? *(const uint4*)(rowp + d0) : make_uint4(0, 0, 0, 0);
-                        S[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lt_v8bf, Qh[ks]), __builtin_bit_cast(lt_v8bf, kf), S[b], 0, 0, 0);
-                        S[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lt_v8bf, Ql[ks]), __builtin_bit_cast(lt_v8bf, kf), S[b], 0, 0, 0);
+                        if ((ks + 1) * 32 > p.key_off) {     // (a step of value-only columns: the query is zero there)
+                            S[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lt_v8bf, Qh[ks]), __builtin_bit_cast(lt_v8bf, kf), S[b], 0, 0, 0);
+                            S[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lt_v8bf, Ql[ks]), __builtin_bit_cast(lt_v8bf, kf), S[b], 0, 0, 0);
+                        }
                         if (d0 < r) {   // the same registers, transposed, are the second product's operand: column d0 + c of key 16 b + n
                             const uint32_t kw[4] = {kf.x, kf.y, kf.z, kf.w};
 #pragma unroll
@@ -474,8 +476,10 @@ __global__ __launch_bounds__(64) void latent_attn_mfma_decode_kernel(const i64h_
                 if (ks * 32 < D) {
                     const int d0 = ks * 32 + kg * 8;
                     const uint4 f = kf[b][ks];
-                    S[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lt_v8bf, Qh[ks]), __builtin_bit_cast(lt_v8bf, f), S[b], 0, 0, 0);
-                    S[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lt_v8bf, Ql[ks]), __builtin_bit_cast(lt_v8bf, f), S[b], 0, 0, 0);
+                    if ((ks + 1) * 32 > p.key_off) {     // (a step of value-only columns: the query is zero there)
+                        S[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lt_v8bf, Qh[ks]), __builtin_bit_cast(lt_v8bf, f), S[b], 0, 0, 0);
+                        S[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lt_v8bf, Ql[ks]), __builtin_bit_cast(lt_v8bf, f), S[b], 0, 0, 0);
+                    }
                     if (d0 < r) {
                         const uint32_t kw[4] = {f.x, f.y, f.z, f.w};
 #pragma unroll
@@ -623,6 +627,7 @@ int i64h_latent_attn(const i64h_latent_attn_args* dp, void* stream) {
     I64H_CHECK_ARG(d.kv_rank <= 64 * LT_MAXC, "latent_attn: kv_rank %d above %d", d.kv_rank, 64 * LT_MAXC);
     I64H_CHECK_ARG(d.cache_dtype == 0 || d.cache_dtype == 2, "latent_attn: cache dtype %d", d.cache_dtype);
     I64H_CHECK_ARG(d.Q && d.cache && d.block_table && d.slot_ids && d.positions && d.out, "latent_attn: null operand");
+    I64H_CHECK_ARG(d.key_off >= 0 && d.key_off <= d.kv_rank, "latent_attn: %d value-only columns of %d value columns", d.key_off, d.kv_rank);
     if (d.n == 0) return 0;
     const int D = d.kv_rank + d.rot_dim;
     const bool mfma_ok = d.cache_dtype == 2 && D % 8 == 0 && d.kv_rank % 16 == 0 && d.kv_rank <= 16 * LT_NB && D <= 32 * LT_KD &&

@@ -162,3 +162,59 @@ def make_dogalorn_weights(cfg, seed: int = 0, std: float = 0.02) -> Dict[str, to
         if L.mlp is not None:
             w.update({p + "mlp.up": rn(L.mlp.ff, W), p + "mlp.up.b": zero(L.mlp.ff), p + "mlp.down": rn(W, L.mlp.ff), p + "mlp.down.b": zero(W)})
     return w
+
+
+def zabutar_config(width: int = 1024, blocks: int = 4, rec_heads: int = 8, rec_dim: int = 128, rec_vdim: int = 128, heads: int = 16, kv_heads: int = 4, dim: int = 64,
+                   vdim: int = 64, ff: int = 4096, experts: int = 8, top: int = 2, expert_ff: int = 1024, identity: int = 2, groups: int = 2, keep: int = 1,
+                   shared_ff: int = 1024, taps: int = 4, vocab: int = 32000, max_positions: int = 4096, rel_rows: int = 32):
+    """A Zabutar configuration with layers of a real model's proportions: `blocks` times (recurrent layer with a dense feed-forward,
+    attention layer with a mixture of experts, recurrent layer with a mixture, attention layer over the first one's keys and values
+    with a dense feed-forward); random weights: make_zabutar_weights."""
+    from .config import ZabutarConfig
+    dense = {"kind": "dense", "ff": ff}
+    moe = {"kind": "moe", "expert": {"ff": expert_ff}, "shared": {"ff": shared_ff},
+           "router": {"experts": experts, "top": top, "identity": identity, "scale": 1.0, "groups": {"count": groups, "keep": keep}}}
+    rec = {"type": "hgrn2", "mixer": {"heads": rec_heads, "dim": rec_dim, "vdim": rec_vdim}}
+    att = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5, "bias_max": float(max_positions)}
+    layers = []
+    for b in range(blocks):
+        layers += [dict(rec, mlp=dense), {"type": "attention", "mixer": dict(att), "mlp": moe}, dict(rec, mlp=moe),
+                   {"type": "attention", "mixer": dict(att, kv_from=4 * b + 1), "mlp": dense}]
+    cfg = ZabutarConfig.from_dict({"architecture": "Zabutar", "vocab": vocab, "width": width, "max_positions": max_positions, "norm": {"eps": 1e-6},
+                                   "canon": {"taps": taps}, "layers": layers})
+    cfg.rel_rows = rel_rows
+    return cfg
+
+
+def make_zabutar_weights(cfg, seed: int = 0, std: float = 0.02) -> Dict[str, torch.Tensor]:
+    """bf16 N(0, std) matrices, norm offsets and biases 0, convolution taps small, gate bounds spread over [0, 0.9], distance bias 0,
+    a router wide enough that the experts' loads differ from token to token."""
+    g = torch.Generator().manual_seed(seed)
+    W = cfg.width
+
+    def rn(*shape, s=std):
+        return torch.empty(*shape, dtype=torch.float32).normal_(0.0, s, generator=g).to(torch.bfloat16)
+
+    zero = lambda *n: torch.zeros(*n, dtype=torch.bfloat16)
+    w = {"embed": rn(cfg.vocab, W), "pos": rn(cfg.max_positions, W), "head": rn(cfg.vocab, W), "final.norm": zero(W)}
+    for i, L in enumerate(cfg.layers):
+        p, m, f = f"l{i}.", L.mixer, L.mlp
+        for q in (1, 2) if f is not None else (1,):
+            w.update({f"{p}norm{q}": zero(W), f"{p}norm{q}b": zero(W), f"{p}canon{q}": rn(W, cfg.canon_taps, s=0.1)})
+        if L.type == "hgrn2":
+            nk, nv = m.heads * m.dim, m.heads * m.vdim
+            w.update({p + "mix.q": rn(nk, W), p + "mix.f": rn(nk, W), p + "mix.f.b": zero(nk), p + "mix.lower": (torch.rand(nk, generator=g) * 0.9).to(torch.bfloat16),
+                      p + "mix.v": rn(nv, W), p + "mix.norm": torch.ones(m.vdim, dtype=torch.bfloat16), p + "mix.o": rn(W, nv)})
+        else:
+            w.update({p + "mix.q": rn(m.heads * m.dim, W), p + "mix.rel": zero(getattr(cfg, "rel_rows", 32), m.heads), p + "mix.o": rn(W, m.heads * m.vdim)})
+            if m.kv_from is None:
+                w.update({p + "mix.k": rn(m.kv_heads * m.dim, W), p + "mix.v": rn(m.kv_heads * m.vdim, W)})
+        if f is not None and f.kind == "dense":
+            w.update({p + "mlp.up": rn(f.ff, W), p + "mlp.up.b": zero(f.ff), p + "mlp.down": rn(W, f.ff), p + "mlp.down.b": zero(W), p + "mlp.act": zero(2)})
+        elif f is not None:
+            w.update({p + "mlp.router": rn(f.entries, W, s=0.1), p + "mlp.correction": zero(f.entries)})
+            for e in range(f.experts):
+                w.update({f"{p}mlp.e{e}.gate": rn(f.ff, W), f"{p}mlp.e{e}.up": rn(f.ff, W), f"{p}mlp.e{e}.down": rn(W, f.ff)})
+            if f.shared_ff:
+                w.update({p + "mlp.shared.gate": rn(f.shared_ff, W), p + "mlp.shared.up": rn(f.shared_ff, W), p + "mlp.shared.down": rn(W, f.shared_ff)})
+    return w
