@@ -33,7 +33,8 @@ int i64h_device_check(void);
  *   bias (may be NULL; fp32 [N], batch stride bias_batch) is added to the sum before any epilogue but the two gate / up ones.
  * group_off (may be NULL; device int32 [batch + 1], ascending): batch b takes the rows [group_off[b], group_off[b + 1]) of a_rows
  *   (of A itself without a_rows) and of C instead of all M rows; M is then the most rows any batch may have (it sizes the launch,
- *   workgroups past a batch's rows leave at once), and the launch needs no count on the host.  Such launches take the 64 x 64 tile form.
+ *   workgroups past a batch's rows leave at once), and the launch needs no count on the host.  Such launches take the 64 x 64 tile form,
+ *   or with M <= 64 the fragment-streaming form.
  * Any M, N, K >= 1; 16-byte loads are used where strides and addresses allow, element loads otherwise.
  * Launches with M <= I64H_SKINNY_ROWS take a weight-streaming form (one wave per output column group). */
 #define I64H_EPI_STORE 0
@@ -249,6 +250,8 @@ typedef struct {
     int64_t ldo;
     int64_t n;
     int32_t mode;
+    int32_t single_rows; /* 1: every row is the only row of its sequence in this launch: the launch that computes a row also stores its
+                            sequence's new carried inputs (no second launch) */
 } i64h_causal_conv_args;
 int i64h_causal_conv(const i64h_causal_conv_args* d, void* stream);
 
@@ -417,6 +420,8 @@ typedef struct {
     float* out;          /* fp32 [n, heads * vdim], row stride ldo */
     int64_t ldo;
     int64_t n;
+    int32_t gates;       /* i64h_gla_scan: 1 = P holds the raw projections and the scan applies i64h_gla_gates' functions as it loads them (P stays
+                            as it is); meant for launches of single rows, where the separate pass would be one more launch for little work */
 } i64h_gla_args;
 int i64h_gla_gates(const i64h_gla_args* d, void* stream);
 int i64h_gla_scan(const i64h_gla_args* d, void* stream);

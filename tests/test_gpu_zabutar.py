@@ -164,7 +164,7 @@ def test_linear_activation_epilogues(dev, epi, M, exact):
 
 
 @pytest.mark.parametrize("exact", [False, True])
-@pytest.mark.parametrize("counts", [[3, 0, 70, 1], [0, 0, 5], [130], [64, 64, 1, 0, 0, 9]])
+@pytest.mark.parametrize("counts", [[3, 0, 70, 1], [0, 0, 5], [130], [64, 64, 1, 0, 0, 9], [17, 0, 33, 2]])
 def test_linear_over_groups_of_rows_counted_on_the_device(dev, exact, counts):
     """Every group multiplies its own rows (gathered through a row list) by its own weight; empty groups, groups longer than a tile."""
     from vllm_i64_amd import ops_dense as D
@@ -234,7 +234,8 @@ def test_input_convolution_under_cuts(dev, taps, cut_sizes):
         r = Rows(dev, runs)
         x = torch.cat([h[s][p:p + c] for s, p, c in runs]).to(dev).contiguous()
         out = torch.empty(r.n, W, device=dev)
-        D.causal_conv(x, off=0, channels=W, w=w.to(dev), bias=None, positions=r.pos, slot_ids=r.slots, state=state, out=out, n=r.n, added=True)
+        single = all(c == 1 for _, _, c in runs)        # (as the runner does: single rows store their carried inputs in the same launch)
+        D.causal_conv(x, off=0, channels=W, w=w.to(dev), bias=None, positions=r.pos, slot_ids=r.slots, state=state, out=out, n=r.n, added=True, single_rows=single)
         row = 0
         for s, p, c in runs:
             got[s].append(out[row:row + c].cpu())
@@ -260,9 +261,11 @@ def _hgrn2_run(dev, w, H, d, dv, h, lens_cuts, eps, state):
         x = torch.cat([h[s][p:p + c] for s, p, c in runs]).double()
         P = torch.cat([x @ w["q"].double().T, x @ w["f"].double().T + w["f.b"].double(), x @ w["v"].double().T], 1).float().to(dev).contiguous()
         cols = dict(q_off=0, f_off=nk, v_off=2 * nk, heads=H, dim=d, vdim=dv, n=r.n)
-        D.gla_gates(P, lower=w["lower"].to(dev), q_act=True, **cols)
+        single = all(c == 1 for _, _, c in runs)        # (as the runner does: single rows have their gate functions applied by the scan)
+        if not single:
+            D.gla_gates(P, lower=w["lower"].to(dev), q_act=True, **cols)
         O, G = torch.empty(r.n, nv, device=dev), torch.empty(r.n, nv, device=dev)
-        D.gla_scan(P, seg_start=r.seg, nseg=r.nseg, positions=r.pos, slot_ids=r.slots, state=state, out=O, **cols)
+        D.gla_scan(P, seg_start=r.seg, nseg=r.nseg, positions=r.pos, slot_ids=r.slots, state=state, out=O, gates=single, lower=w["lower"].to(dev), q_act=True, **cols)
         D.gate_norm(O, w["norm"].repeat(H).to(dev), G, groups=H, eps=eps, n=r.n)
         row = 0
         for s, p, c in runs:

@@ -66,6 +66,9 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(const i64h_gla_args p, co
         }
     }
     const int qoff = p.q_off + a * N + n0, foff = p.f_off + a * N + n0, koff = HASK ? p.k_off + a * N + n0 : 0;
+    float low[KPT];     // the gates' lower bounds, where the scan applies the gate functions itself
+#pragma unroll
+    for (int k = 0; k < KPT; ++k) low[k] = (p.gates && p.lower && n0 + k < N) ? p.lower[a * N + n0 + k] : 0.0f;
     struct Tok {
         float q[KPT], f[KPT], k[HASK ? KPT : 1], v[CPT];
     };
@@ -92,6 +95,13 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(const i64h_gla_args p, co
                 u.q[k] = ok ? row[qoff + k] : 0.0f;
                 u.f[k] = ok ? row[foff + k] : 1.0f;
                 if (HASK) u.k[k] = ok ? row[koff + k] : 0.0f;
+            }
+        }
+        if (p.gates) {
+#pragma unroll
+            for (int k = 0; k < KPT; ++k) {
+                if (p.q_act) u.q[k] = u.q[k] * bl_sigmoid(u.q[k]);
+                u.f[k] = n0 + k < N ? low[k] + (1.0f - low[k]) * bl_sigmoid(u.f[k]) : 1.0f;
             }
         }
 #pragma unroll

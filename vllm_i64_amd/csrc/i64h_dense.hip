@@ -405,7 +405,14 @@ __global__ __launch_bounds__(64 * NW) void linear_rows64_kernel(const i64h_linea
     const int n = lane & 15, kg = lane >> 4;
     const int64_t b = blockIdx.z;
     const int n0 = blockIdx.x * 16;
-    const int M = (int)p.M, N = p.N, K = p.K;
+    int M = (int)p.M;
+    const int N = p.N, K = p.K;
+    int64_t g0 = 0;      // this batch's first row among all rows, where the rows are dealt to the batches by group_off
+    if (p.group_off) {
+        g0 = p.group_off[b];
+        M = min(M, p.group_off[b + 1] - (int)g0);
+        if (M <= 0) return;
+    }
     const int mblocks = (M + 15) / 16;
     const bool cok = n0 + n < N;
     const uint16_t* pw = (const uint16_t*)p.W + b * p.w_batch + (int64_t)(cok ? n0 + n : 0) * K;
@@ -416,7 +423,7 @@ __global__ __launch_bounds__(64 * NW) void linear_rows64_kernel(const i64h_linea
     for (int i = 0; i < 4; ++i) {
         const int m = i * 16 + n;
         rok[i] = m < M;
-        const int64_t arow = rok[i] ? (p.a_rows ? (int64_t)p.a_rows[m] : m) : 0;
+        const int64_t arow = rok[i] ? (p.a_rows ? (int64_t)p.a_rows[g0 + m] : g0 + m) : 0;
         pa[i] = p.A + b * p.a_batch + arow * p.lda;
     }
     dn_v4f acc[4], acc2[4];
@@ -481,7 +488,7 @@ __global__ __launch_bounds__(64 * NW) void linear_rows64_kernel(const i64h_linea
             s += red[0][w][m][c];
             if (DUAL) s2 += red[DUAL ? 1 : 0][w][m][c];
         }
-        C[(int64_t)m * p.ldc + n0 + c] = dn_epilogue<EPI>(p, s, s2, b, m, n0 + c);
+        C[(g0 + m) * p.ldc + n0 + c] = dn_epilogue<EPI>(p, s, s2, b, g0 + m, n0 + c);
     }
 }
 
@@ -736,7 +743,7 @@ int i64h_linear_run(const i64h_linear* dp, void* stream) {
         I64H_CHECK_LAUNCH();
         return 0;
     }
-    if (g_rows64 && !d.group_off && !d.exact && d.M <= 64 && vecA && vecW) {
+    if (g_rows64 && !d.exact && d.M <= 64 && vecA && vecW) {
         const dim3 grid((unsigned)((d.N + 15) / 16), 1, (unsigned)d.batch);
         switch (d.epilogue) {
             // eight waves share the k steps where one accumulator is kept (the gate / up pair needs twice the LDS: four)

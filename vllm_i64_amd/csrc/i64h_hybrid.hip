@@ -64,6 +64,7 @@ __global__ __launch_bounds__(256) void prev_token_kernel(const i64h_embed_bigram
 
 // ---------------------------------------------------------------------------------------------------------------------------
 #define HY_MAX_STREAMS 8
+#define HY_MAX_TAPS 16
 __global__ __launch_bounds__(256) void streams_kernel(const i64h_streams_args p) {
     extern __shared__ float sv[];   // [W] the weighted read of the row, then 4 floats for reductions
     const int tid = threadIdx.x;
@@ -159,6 +160,13 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(const i64h_causal_conv
     const float x = p.P[t * p.ldp + p.off + c];
     a += p.w[(int64_t)c * p.taps + p.taps - 1] * x;
     p.out[t * p.ldo + c] = p.mode == 1 ? x + a : hy_silu(a);
+    if (p.single_rows && p.taps > 1) {      // no other row of the launch reads or writes this sequence's carried inputs
+        float v[HY_MAX_TAPS];
+        for (int d = 1; d < p.taps - 1; ++d) v[d] = conv_input(p, t, d, before, c);
+        float* st = p.state + (int64_t)p.slot_ids[t] * (p.taps - 1) * p.channels + c;
+        for (int d = 1; d < p.taps - 1; ++d) st[(int64_t)(p.taps - 2 - d) * p.channels] = v[d];
+        st[(int64_t)(p.taps - 2) * p.channels] = x;
+    }
 }
 
 // the same for 2 .. 8 taps: a thread walks CV_ROWS consecutive rows of its channel with the weights and the last TAPS - 1 inputs in
@@ -191,7 +199,6 @@ __global__ __launch_bounds__(256) void causal_conv_walk_kernel(const i64h_causal
     }
 }
 
-#define HY_MAX_TAPS 16
 __global__ __launch_bounds__(256) void conv_carry_kernel(const i64h_causal_conv_args p) {
     const int64_t t = blockIdx.y;
     const int c = blockIdx.x * 256 + threadIdx.x;
@@ -575,7 +582,7 @@ int i64h_causal_conv(const i64h_causal_conv_args* dp, void* stream) {
     const dim3 grid((unsigned)((d.channels + 255) / 256), (unsigned)d.n);
     const dim3 walk((unsigned)((d.channels + 255) / 256), (unsigned)((d.n + CV_ROWS - 1) / CV_ROWS));
     hipStream_t s = (hipStream_t)stream;
-    switch (d.n >= 32 * CV_ROWS ? d.taps : 0) {     // few rows: a thread per row and channel fills the chip better
+    switch ((d.n >= 32 * CV_ROWS && !d.single_rows) ? d.taps : 0) {     // few rows: a thread per row and channel fills the chip better
         case 2: hipLaunchKernelGGL(causal_conv_walk_kernel<2>, walk, dim3(256), 0, s, d); break;
         case 3: hipLaunchKernelGGL(causal_conv_walk_kernel<3>, walk, dim3(256), 0, s, d); break;
         case 4: hipLaunchKernelGGL(causal_conv_walk_kernel<4>, walk, dim3(256), 0, s, d); break;
@@ -586,7 +593,7 @@ int i64h_causal_conv(const i64h_causal_conv_args* dp, void* stream) {
         default: hipLaunchKernelGGL(causal_conv_kernel, grid, dim3(256), 0, s, d); break;
     }
     I64H_CHECK_LAUNCH();
-    if (d.taps > 1) {
+    if (d.taps > 1 && !d.single_rows) {
         hipLaunchKernelGGL(conv_carry_kernel, grid, dim3(256), 0, (hipStream_t)stream, d);
         I64H_CHECK_LAUNCH();
     }

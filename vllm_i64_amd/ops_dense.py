@@ -212,9 +212,11 @@ def streams_step(streams: torch.Tensor, *, y: Optional[torch.Tensor] = None, y2:
 
 
 def causal_conv(p: torch.Tensor, *, off: int, channels: int, w: torch.Tensor, bias: Optional[torch.Tensor], positions: torch.Tensor,
-                slot_ids: torch.Tensor, state: Optional[torch.Tensor], out: torch.Tensor, n: Optional[int] = None, added: bool = False) -> torch.Tensor:
+                slot_ids: torch.Tensor, state: Optional[torch.Tensor], out: torch.Tensor, n: Optional[int] = None, added: bool = False,
+                single_rows: bool = False) -> torch.Tensor:
     """See i64h_causal_conv.  p fp32 [n, ldp]; w fp32 [channels, taps]; state fp32 [slots, taps - 1, channels]; out fp32 [n, channels].
-    added: the convolution is added to its own input and no activation follows (mode 1)."""
+    added: the convolution is added to its own input and no activation follows (mode 1).  single_rows: the caller vouches that every row
+    is the only row of its sequence in this launch; the carried inputs are then stored by the same launch."""
     _chk(p, torch.float32, "p"), _chk(w, torch.float32, "w"), _chk(out, torch.float32, "out")
     _chk(positions, torch.int32, "positions"), _chk(slot_ids, torch.int32, "slot_ids")
     rows = int(n if n is not None else positions.numel())
@@ -231,7 +233,7 @@ def causal_conv(p: torch.Tensor, *, off: int, channels: int, w: torch.Tensor, bi
             (bias is not None and bias.numel() != channels) or (taps > 1 and (state.shape[-1] != channels or state.shape[-2] != taps - 1)):
         raise _lib.I64HError("causal_conv: shapes do not fit the sizes")
     d = _lib.CausalConv(P=ptr(p), ldp=p.shape[-1], off=off, channels=channels, taps=taps, w=ptr(w), bias=ptr(bias), positions=ptr(positions),
-                        slot_ids=ptr(slot_ids), state=ptr(state), out=ptr(out), ldo=channels, n=rows, mode=1 if added else 0)
+                        slot_ids=ptr(slot_ids), state=ptr(state), out=ptr(out), ldo=channels, n=rows, mode=1 if added else 0, single_rows=int(bool(single_rows)))
     call_dense("i64h_causal_conv", _ref(d), _stream())
     return out
 
@@ -395,15 +397,18 @@ def gla_gates(p: torch.Tensor, *, q_off: int, f_off: int, v_off: int, heads: int
 
 
 def gla_scan(p: torch.Tensor, *, q_off: int, f_off: int, v_off: int, heads: int, dim: int, vdim: int, seg_start: torch.Tensor, nseg: int,
-             positions: torch.Tensor, slot_ids: torch.Tensor, state: torch.Tensor, out: torch.Tensor, n: int, k_off: int = -1) -> torch.Tensor:
-    """See i64h_gla_scan.  state fp32 [slots, heads, vdim, dim]; out fp32 [n, heads * vdim]; k_off < 0: the key is one minus the decay."""
+             positions: torch.Tensor, slot_ids: torch.Tensor, state: torch.Tensor, out: torch.Tensor, n: int, k_off: int = -1,
+             gates: bool = False, lower: Optional[torch.Tensor] = None, q_act: bool = False) -> torch.Tensor:
+    """See i64h_gla_scan.  state fp32 [slots, heads, vdim, dim]; out fp32 [n, heads * vdim]; k_off < 0: the key is one minus the decay.
+    gates: p holds the raw projections and the scan applies gla_gates' functions (lower, q_act) as it loads them."""
     _chk(state, torch.float32, "state"), _chk(out, torch.float32, "out")
     _chk(seg_start, torch.int32, "seg_start"), _chk(positions, torch.int32, "positions"), _chk(slot_ids, torch.int32, "slot_ids")
     _rows_ok("gla_scan", n, positions, slot_ids)
     if tuple(state.shape[1:]) != (heads, vdim, dim) or out.numel() < n * heads * vdim or seg_start.numel() < nseg + 1:
         raise _lib.I64HError("gla_scan: shapes do not fit the sizes")
     d = _gla_args(p, q_off=q_off, f_off=f_off, v_off=v_off, heads=heads, dim=dim, vdim=vdim, k_off=k_off, n=n, seg_start=ptr(seg_start), nseg=nseg,
-                  positions=ptr(positions), slot_ids=ptr(slot_ids), state=ptr(state), out=ptr(out), ldo=heads * vdim)
+                  positions=ptr(positions), slot_ids=ptr(slot_ids), state=ptr(state), out=ptr(out), ldo=heads * vdim, gates=int(bool(gates)),
+                  lower=lower if gates else None, q_act=bool(q_act) and bool(gates))
     call_dense("i64h_gla_scan", _ref(d), _stream())
     return out
 

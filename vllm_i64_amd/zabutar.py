@@ -221,15 +221,17 @@ class ZabutarModel:
         return torch.tensor(starts, dtype=torch.int32).to(self.device), len(starts) - 1
 
     # ---- mixers and feed-forwards: the sublayer input is B.hc; the result lands in B.y ----
-    def _hgrn2(self, B, d, l, n, positions, slot_ids, kvc, seg, nseg) -> None:
+    def _hgrn2(self, B, d, l, n, positions, slot_ids, kvc, seg, nseg, single) -> None:
         m, ex = d["m"], self.exact
         nk, nv = m.heads * m.dim, m.heads * m.vdim
         P = B.p[: n * d["n_in"]].view(n, d["n_in"])
         D.linear(B.hc, d["w_in"], P, exact=ex, bias=d["b_in"])
         cols = dict(q_off=0, f_off=nk, v_off=2 * nk, heads=m.heads, dim=m.dim, vdim=m.vdim, n=n)
-        D.gla_gates(P, lower=d["lower"], q_act=True, **cols)
+        if not single:      # (single rows: the scan applies the gate functions itself, one launch less)
+            D.gla_gates(P, lower=d["lower"], q_act=True, **cols)
         O = B.a[: n * nv].view(n, nv)
-        D.gla_scan(P, seg_start=seg, nseg=nseg, positions=positions, slot_ids=slot_ids, state=kvc.state[l]["gla"], out=O, **cols)
+        D.gla_scan(P, seg_start=seg, nseg=nseg, positions=positions, slot_ids=slot_ids, state=kvc.state[l]["gla"], out=O, gates=single, lower=d["lower"],
+                   q_act=True, **cols)
         G = B.b[: n * nv].view(n, nv)
         D.gate_norm(O, d["norm"], G, groups=m.heads, eps=self.cfg.norm_eps, n=n)
         D.linear(G, d["o"], B.y, exact=ex)
@@ -311,6 +313,8 @@ class ZabutarModel:
             runs = attention_segments(tokens_per_seq, n, self.ATTN_MAX_SEGMENTS)
         else:
             runs = [(0, n, bool(rows_are_slots))]
+        # every row the only row of its sequence (a decode step): kernels that keep per-sequence state may then store it in the launch that reads it
+        single = bool(rows_are_slots) or (tokens_per_seq is not None and all(int(t) <= 1 for t in tokens_per_seq))
         D.embed_bigram(token_ids, positions, slot_ids, self.embed, B.streams, pos_table=self.pos)
         # every residual launch adds the normed result of the sublayer before it and norms for the sublayer after it
         D.streams_step(B.streams, norm_w=self.layers[0]["norm1"], eps=eps, h=B.h)
@@ -318,13 +322,13 @@ class ZabutarModel:
         for i, (l, q) in enumerate(subs):
             d = self.layers[l]
             D.causal_conv(B.h, off=0, channels=cfg.width, w=d[f"canon{q}"], bias=None, positions=positions, slot_ids=slot_ids,
-                          state=kvc.state[l].get(f"canon{q}"), out=B.hc, n=n, added=True)
+                          state=kvc.state[l].get(f"canon{q}"), out=B.hc, n=n, added=True, single_rows=single)
             if q == 2 and d["mlp"].kind == "dense":
                 self._dense_ff(B, d, n)
             elif q == 2:
                 self._moe_ff(B, d, n, record, l)
             elif d["type"] == "hgrn2":
-                self._hgrn2(B, d, l, n, positions, slot_ids, kvc, seg, nseg)
+                self._hgrn2(B, d, l, n, positions, slot_ids, kvc, seg, nseg, single)
             else:
                 self._attention(B, d, l, n, positions, slot_ids, kvc, runs, int(max_ctx_hint))
             write = dict(y=B.y, yn_w=d[f"norm{q}b"], y_eps=eps, out_w=self.ones1)
