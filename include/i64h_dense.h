@@ -420,8 +420,6 @@ typedef struct {
     float* out;          /* fp32 [n, heads * vdim], row stride ldo */
     int64_t ldo;
     int64_t n;
-    int32_t gates;       /* i64h_gla_scan: 1 = P holds the raw projections and the scan applies i64h_gla_gates' functions as it loads them (P stays
-                            as it is); meant for launches of single rows, where the separate pass would be one more launch for little work */
 } i64h_gla_args;
 int i64h_gla_gates(const i64h_gla_args* d, void* stream);
 int i64h_gla_scan(const i64h_gla_args* d, void* stream);

@@ -261,11 +261,9 @@ def _hgrn2_run(dev, w, H, d, dv, h, lens_cuts, eps, state):
         x = torch.cat([h[s][p:p + c] for s, p, c in runs]).double()
         P = torch.cat([x @ w["q"].double().T, x @ w["f"].double().T + w["f.b"].double(), x @ w["v"].double().T], 1).float().to(dev).contiguous()
         cols = dict(q_off=0, f_off=nk, v_off=2 * nk, heads=H, dim=d, vdim=dv, n=r.n)
-        single = all(c == 1 for _, _, c in runs)        # (as the runner does: single rows have their gate functions applied by the scan)
-        if not single:
-            D.gla_gates(P, lower=w["lower"].to(dev), q_act=True, **cols)
+        D.gla_gates(P, lower=w["lower"].to(dev), q_act=True, **cols)
         O, G = torch.empty(r.n, nv, device=dev), torch.empty(r.n, nv, device=dev)
-        D.gla_scan(P, seg_start=r.seg, nseg=r.nseg, positions=r.pos, slot_ids=r.slots, state=state, out=O, gates=single, lower=w["lower"].to(dev), q_act=True, **cols)
+        D.gla_scan(P, seg_start=r.seg, nseg=r.nseg, positions=r.pos, slot_ids=r.slots, state=state, out=O, **cols)
         D.gate_norm(O, w["norm"].repeat(H).to(dev), G, groups=H, eps=eps, n=r.n)
         row = 0
         for s, p, c in runs:

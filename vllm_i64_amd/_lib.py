@@ -323,7 +323,7 @@ class Gla(ctypes.Structure):
     """Mirror of i64h_gla_args (include/i64h_dense.h)."""
     _fields_ = [("P", _P), ("ldp", _L), ("q_off", _I), ("f_off", _I), ("k_off", _I), ("v_off", _I), ("heads", _I), ("dim", _I), ("vdim", _I),
                 ("lower", _P), ("q_act", _I), ("seg_start", _P), ("nseg", _I), ("positions", _P), ("slot_ids", _P), ("state", _P), ("out", _P),
-                ("ldo", _L), ("n", _L), ("gates", _I)]
+                ("ldo", _L), ("n", _L)]
 
 
 class Route(ctypes.Structure):

@@ -31,7 +31,7 @@ __global__ __launch_bounds__(256) void gla_gates_kernel(const i64h_gla_args p) {
 // the same order however a prompt is cut).  Loads run GL_TG tokens ahead in two alternating register sets, so that a wave that is alone
 // on its SIMD still has a group of tokens in flight while it computes one.  State layout [slot, head, value column, key channel].
 #define GL_TG 4
-template <int KPT, int CPT, bool HASK, bool GATES>
+template <int KPT, int CPT, bool HASK>
 __global__ __launch_bounds__(256) void gla_scan_kernel(const i64h_gla_args p, const int ctiles, const int vec) {
     const int N = p.dim, P = p.vdim;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -66,12 +66,6 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(const i64h_gla_args p, co
         }
     }
     const int qoff = p.q_off + a * N + n0, foff = p.f_off + a * N + n0, koff = HASK ? p.k_off + a * N + n0 : 0;
-    float low[GATES ? KPT : 1];     // the gates' lower bounds, where the scan applies the gate functions itself (an instance of its own:
-                                    // the long-run instance keeps its registers for tokens in flight)
-    if (GATES) {
-#pragma unroll
-        for (int k = 0; k < KPT; ++k) low[k] = (p.lower && n0 + k < N) ? p.lower[a * N + n0 + k] : 0.0f;
-    }
     struct Tok {
         float q[KPT], f[KPT], k[HASK ? KPT : 1], v[CPT];
     };
@@ -98,13 +92,6 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(const i64h_gla_args p, co
                 u.q[k] = ok ? row[qoff + k] : 0.0f;
                 u.f[k] = ok ? row[foff + k] : 1.0f;
                 if (HASK) u.k[k] = ok ? row[koff + k] : 0.0f;
-            }
-        }
-        if (GATES) {
-#pragma unroll
-            for (int k = 0; k < KPT; ++k) {
-                if (p.q_act) u.q[k] = u.q[k] * bl_sigmoid(u.q[k]);
-                u.f[k] = n0 + k < N ? low[k] + (1.0f - low[k]) * bl_sigmoid(u.f[k]) : 1.0f;
             }
         }
 #pragma unroll
@@ -325,19 +312,17 @@ int i64h_gla_scan(const i64h_gla_args* dp, void* stream) {
                         (uintptr_t)d.P % 16 == 0 && (uintptr_t)d.state % 16 == 0;
         hipLaunchKernelGGL(kern, grid, dim3(256), 0, (hipStream_t)stream, d, ctiles, vec);
     };
-#define GLA_PICK(C, HK, GT)                                          \
-    if (kpt <= 1) launch(gla_scan_kernel<1, C, HK, GT>, 1);          \
-    else if (kpt <= 2) launch(gla_scan_kernel<2, C, HK, GT>, 2);     \
-    else if (kpt <= 4) launch(gla_scan_kernel<4, C, HK, GT>, 4);     \
-    else if (kpt <= 8) launch(gla_scan_kernel<8, C, HK, GT>, 8);     \
-    else launch(gla_scan_kernel<16, C, HK, GT>, 16);
-#define GLA_PICK2(C, HK) if (d.gates) { GLA_PICK(C, HK, true) } else { GLA_PICK(C, HK, false) }
+#define GLA_PICK(C, HK)                                          \
+    if (kpt <= 1) launch(gla_scan_kernel<1, C, HK>, 1);          \
+    else if (kpt <= 2) launch(gla_scan_kernel<2, C, HK>, 2);     \
+    else if (kpt <= 4) launch(gla_scan_kernel<4, C, HK>, 4);     \
+    else if (kpt <= 8) launch(gla_scan_kernel<8, C, HK>, 8);     \
+    else launch(gla_scan_kernel<16, C, HK>, 16);
     if (cpt == 2) {
-        if (hask) { GLA_PICK2(2, true) } else { GLA_PICK2(2, false) }
+        if (hask) { GLA_PICK(2, true) } else { GLA_PICK(2, false) }
     } else {
-        if (hask) { GLA_PICK2(1, true) } else { GLA_PICK2(1, false) }
+        if (hask) { GLA_PICK(1, true) } else { GLA_PICK(1, false) }
     }
-#undef GLA_PICK2
 #undef GLA_PICK
     I64H_CHECK_LAUNCH();
     return 0;

@@ -397,18 +397,15 @@ def gla_gates(p: torch.Tensor, *, q_off: int, f_off: int, v_off: int, heads: int
 
 
 def gla_scan(p: torch.Tensor, *, q_off: int, f_off: int, v_off: int, heads: int, dim: int, vdim: int, seg_start: torch.Tensor, nseg: int,
-             positions: torch.Tensor, slot_ids: torch.Tensor, state: torch.Tensor, out: torch.Tensor, n: int, k_off: int = -1,
-             gates: bool = False, lower: Optional[torch.Tensor] = None, q_act: bool = False) -> torch.Tensor:
-    """See i64h_gla_scan.  state fp32 [slots, heads, vdim, dim]; out fp32 [n, heads * vdim]; k_off < 0: the key is one minus the decay.
-    gates: p holds the raw projections and the scan applies gla_gates' functions (lower, q_act) as it loads them."""
+             positions: torch.Tensor, slot_ids: torch.Tensor, state: torch.Tensor, out: torch.Tensor, n: int, k_off: int = -1) -> torch.Tensor:
+    """See i64h_gla_scan.  state fp32 [slots, heads, vdim, dim]; out fp32 [n, heads * vdim]; k_off < 0: the key is one minus the decay."""
     _chk(state, torch.float32, "state"), _chk(out, torch.float32, "out")
     _chk(seg_start, torch.int32, "seg_start"), _chk(positions, torch.int32, "positions"), _chk(slot_ids, torch.int32, "slot_ids")
     _rows_ok("gla_scan", n, positions, slot_ids)
     if tuple(state.shape[1:]) != (heads, vdim, dim) or out.numel() < n * heads * vdim or seg_start.numel() < nseg + 1:
         raise _lib.I64HError("gla_scan: shapes do not fit the sizes")
     d = _gla_args(p, q_off=q_off, f_off=f_off, v_off=v_off, heads=heads, dim=dim, vdim=vdim, k_off=k_off, n=n, seg_start=ptr(seg_start), nseg=nseg,
-                  positions=ptr(positions), slot_ids=ptr(slot_ids), state=ptr(state), out=ptr(out), ldo=heads * vdim, gates=int(bool(gates)),
-                  lower=lower if gates else None, q_act=bool(q_act) and bool(gates))
+                  positions=ptr(positions), slot_ids=ptr(slot_ids), state=ptr(state), out=ptr(out), ldo=heads * vdim)
     call_dense("i64h_gla_scan", _ref(d), _stream())
     return out
 

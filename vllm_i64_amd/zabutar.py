@@ -221,17 +221,15 @@ class ZabutarModel:
         return torch.tensor(starts, dtype=torch.int32).to(self.device), len(starts) - 1
 
     # ---- mixers and feed-forwards: the sublayer input is B.hc; the result lands in B.y ----
-    def _hgrn2(self, B, d, l, n, positions, slot_ids, kvc, seg, nseg, single) -> None:
+    def _hgrn2(self, B, d, l, n, positions, slot_ids, kvc, seg, nseg) -> None:
         m, ex = d["m"], self.exact
         nk, nv = m.heads * m.dim, m.heads * m.vdim
         P = B.p[: n * d["n_in"]].view(n, d["n_in"])
         D.linear(B.hc, d["w_in"], P, exact=ex, bias=d["b_in"])
         cols = dict(q_off=0, f_off=nk, v_off=2 * nk, heads=m.heads, dim=m.dim, vdim=m.vdim, n=n)
-        if not single:      # (single rows: the scan applies the gate functions itself, one launch less)
-            D.gla_gates(P, lower=d["lower"], q_act=True, **cols)
+        D.gla_gates(P, lower=d["lower"], q_act=True, **cols)
         O = B.a[: n * nv].view(n, nv)
-        D.gla_scan(P, seg_start=seg, nseg=nseg, positions=positions, slot_ids=slot_ids, state=kvc.state[l]["gla"], out=O, gates=single, lower=d["lower"],
-                   q_act=True, **cols)
+        D.gla_scan(P, seg_start=seg, nseg=nseg, positions=positions, slot_ids=slot_ids, state=kvc.state[l]["gla"], out=O, **cols)
         G = B.b[: n * nv].view(n, nv)
         D.gate_norm(O, d["norm"], G, groups=m.heads, eps=self.cfg.norm_eps, n=n)
         D.linear(G, d["o"], B.y, exact=ex)
@@ -313,7 +311,7 @@ class ZabutarModel:
             runs = attention_segments(tokens_per_seq, n, self.ATTN_MAX_SEGMENTS)
         else:
             runs = [(0, n, bool(rows_are_slots))]
-        # every row the only row of its sequence (a decode step): kernels that keep per-sequence state may then store it in the launch that reads it
+        # every row the only row of its sequence (a decode step): the convolutions then store their carried inputs in the launch that reads them
         single = bool(rows_are_slots) or (tokens_per_seq is not None and all(int(t) <= 1 for t in tokens_per_seq))
         D.embed_bigram(token_ids, positions, slot_ids, self.embed, B.streams, pos_table=self.pos)
         # every residual launch adds the normed result of the sublayer before it and norms for the sublayer after it
@@ -328,7 +326,7 @@ class ZabutarModel:
             elif q == 2:
                 self._moe_ff(B, d, n, record, l)
             elif d["type"] == "hgrn2":
-                self._hgrn2(B, d, l, n, positions, slot_ids, kvc, seg, nseg, single)
+                self._hgrn2(B, d, l, n, positions, slot_ids, kvc, seg, nseg)
             else:
                 self._attention(B, d, l, n, positions, slot_ids, kvc, runs, int(max_ctx_hint))
             write = dict(y=B.y, yn_w=d[f"norm{q}b"], y_eps=eps, out_w=self.ones1)
