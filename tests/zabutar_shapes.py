@@ -37,7 +37,8 @@ def layer(mix, ff):
     return d
 
 
-# nothing equal and nothing a power of two / the branches that a config may leave out / sizes that the matrix-core kernels take
+# nothing equal and nothing a power of two / the branches that a config may leave out / sizes that the matrix-core kernels take /
+# sizes that fit no 16-byte access (width, head sizes and feed-forward sizes that are no multiples of four)
 SHAPES = {
     "odd": {"architecture": "Zabutar", "vocab": 83, "width": 40, "max_positions": 300, "norm": {"eps": 1e-5}, "canon": {"taps": 3},
             "layers": [layer(hgrn(3, 10, 6), dense(36)),
@@ -49,6 +50,9 @@ SHAPES = {
     "plain": {"architecture": "Zabutar", "vocab": 64, "width": 32, "max_positions": 256, "norm": {"eps": 1e-6}, "canon": {"taps": 1},
               "layers": [layer(attn(1, 1, 16, 16, bias_max=40, rel_rows=6), dense(48)), layer(hgrn(1, 8, 8), None),
                          layer(attn(2, 1, 16, 16, bias_max=3, rel_rows=2, kv_from=0), moe(16, 2, 2, shared=16))]},
+    "ragged": {"architecture": "Zabutar", "vocab": 51, "width": 42, "max_positions": 200, "norm": {"eps": 1e-6}, "canon": {"taps": 2},
+               "layers": [layer(attn(3, 1, 6, 10, rel_rows=3, bias_max=7), moe(10, 3, 2, shared=6)), layer(hgrn(2, 9, 7), dense(30)),
+                          layer(attn(3, 1, 6, 10, rel_rows=5, bias_max=19, kv_from=0), dense(18)), layer(hgrn(1, 17, 3), None)]},
     "wide": {"architecture": "Zabutar", "vocab": 200, "width": 128, "max_positions": 512, "norm": {"eps": 1e-6}, "canon": {"taps": 5},
              "layers": [layer(hgrn(4, 64, 32), moe(48, 16, 4, groups=(4, 2), scale=1.3, shared=96)),
                         layer(attn(8, 2, 64, 64, rel_rows=32, bias_max=48), dense(160)),

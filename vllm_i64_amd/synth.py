@@ -165,7 +165,7 @@ def make_dogalorn_weights(cfg, seed: int = 0, std: float = 0.02) -> Dict[str, to
 
 
 def zabutar_config(width: int = 1024, blocks: int = 4, rec_heads: int = 8, rec_dim: int = 128, rec_vdim: int = 128, heads: int = 16, kv_heads: int = 4, dim: int = 64,
-                   vdim: int = 64, ff: int = 4096, experts: int = 8, top: int = 2, expert_ff: int = 1024, identity: int = 2, groups: int = 2, keep: int = 1,
+                   vdim: int = 64, ff: int = 4096, experts: int = 8, top: int = 2, expert_ff: int = 1024, identity: int = 0, groups: int = 4, keep: int = 2,
                    shared_ff: int = 1024, taps: int = 4, vocab: int = 32000, max_positions: int = 4096, rel_rows: int = 32):
     """A Zabutar configuration with layers of a real model's proportions: `blocks` times (recurrent layer with a dense feed-forward,
     attention layer with a mixture of experts, recurrent layer with a mixture, attention layer over the first one's keys and values

@@ -272,7 +272,7 @@ class ZabutarModel:
         f, ex, W = d["mlp"], self.exact, self.cfg.width
         E, top = f.experts, f.top
         logits = B.act[: n * f.entries].view(n, f.entries)
-        D.linear(B.hc, d["router"], logits, exact=ex)
+        D.linear(B.hc, d["router"], logits, exact=True)      # the router's products in 32 bits in both modes: a choice is not rounding's to make
         D.route_topk(logits, entries=f.entries, correction=d["correction"], groups=f.groups, keep=f.keep, top=top, scale=f.scale, idx=B.idx, wgt=B.wgt, n=n)
         if record is not None:
             record[f"l{l}.route"] = B.idx[: n * top].view(n, top).clone()
