@@ -439,6 +439,10 @@ typedef struct {
     int32_t* idx;
     float* wgt;
     int64_t n;
+    const float* h;
+    int64_t ldh;
+    const void* W;
+    int32_t K;
 } i64h_route_args;
 int i64h_route_topk(const i64h_route_args* d, void* stream);
 

@@ -514,6 +514,14 @@ def test_router_choices_and_weights(dev, E, groups, keep, top):
     D.route_topk(z.to(dev), entries=E, correction=corr.to(dev), groups=groups, keep=keep, top=top, scale=1.7, idx=gi, wgt=gw, n=n)
     assert torch.equal(gi.cpu().long(), idx)          # the same entries in the same order (largest first)
     assert close(gw, wgt, 1e-5)
+    # the launch that computes the logits itself, in 32 bits, from the router's input and weight (column counts with and without 16-byte rows)
+    for K in (72, 45):
+        h = torch.randn(n, K, generator=g)
+        w = (torch.randn(E, K, generator=g) * 2 * K ** -0.5).to(torch.bfloat16)
+        idx, wgt = R.route(h.double() @ w.double().T, corr.double(), r)
+        D.route_topk(None, h=h.to(dev), w=w.to(dev), entries=E, correction=corr.to(dev), groups=groups, keep=keep, top=top, scale=1.7, idx=gi, wgt=gw, n=n)
+        same = (gi.cpu().long() == idx).all(-1)
+        assert float(same.double().mean()) > 0.99 and close(gw.cpu()[same], wgt[same], 1e-4)      # (a close call in 32 bits may fall the other way)
 
 
 @pytest.mark.parametrize("name,l", [("odd", 1), ("odd", 3), ("odd", 5), ("plain", 2), ("wide", 0), ("wide", 2)])

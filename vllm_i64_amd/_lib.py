@@ -329,7 +329,7 @@ class Gla(ctypes.Structure):
 class Route(ctypes.Structure):
     """Mirror of i64h_route_args (include/i64h_dense.h)."""
     _fields_ = [("logits", _P), ("ld", _L), ("E", _I), ("correction", _P), ("groups", _I), ("keep", _I), ("top", _I), ("scale", _F), ("idx", _P),
-                ("wgt", _P), ("n", _L)]
+                ("wgt", _P), ("n", _L), ("h", _P), ("ldh", _L), ("W", _P), ("K", _I)]
 
 
 class MoePlan(ctypes.Structure):

@@ -384,11 +384,11 @@ def _zabutar_kernels(sz, rows, batch, ctx, dev):
         row(f"dogalorn_linear_up_bias_gelu_{tag}", t, flops=2.0 * n * ff * W, bytes_=2.0 * ff * W + 4.0 * n * (W + ff))
         # mixture of experts: router choice, grouping, the two grouped Linears, the weighted sum (beside the dense gate / up pair of equal work)
         ent = E
-        logits = rn(n, ent) * 2
+        w_r = (rn(ent, W) * 0.1).to(torch.bfloat16)
         idx, wgt = torch.empty(n, top, dtype=torch.int32, device=dev), torch.empty(n, top, device=dev)
         corr = torch.zeros(ent, device=dev)
-        t = _time(lambda: D.route_topk(logits, entries=ent, correction=corr, groups=4, keep=2, top=top, scale=1.0, idx=idx, wgt=wgt, n=n), reps)
-        row(f"route_topk_{tag}", t, bytes_=4.0 * n * (ent + 2 * top))
+        t = _time(lambda: D.route_topk(None, h=a, w=w_r, entries=ent, correction=corr, groups=4, keep=2, top=top, scale=1.0, idx=idx, wgt=wgt, n=n), reps)
+        row(f"route_topk_{tag}", t, bytes_=4.0 * n * (W + 2 * top) + 2.0 * ent * W)
         goff, ptok, prow = torch.empty(E + 1, dtype=torch.int32, device=dev), torch.empty(n * top, dtype=torch.int32, device=dev), torch.empty(n * top, dtype=torch.int32, device=dev)
         t = _time(lambda: D.moe_plan(idx, n=n, top=top, experts=E, group_off=goff, pair_token=ptok, pair_row=prow), reps)
         row(f"moe_plan_{tag}", t, bytes_=4.0 * n * top * 3)

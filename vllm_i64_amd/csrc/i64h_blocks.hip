@@ -160,13 +160,51 @@ __global__ __launch_bounds__(256) void route_topk_kernel(const i64h_route_args p
     volatile float* sc = rt_lds + (size_t)wid * (2 * E + G);
     volatile float* ch = sc + E;
     volatile float* gflag = ch + E;
-    const float* z = p.logits + t * p.ld;
+    if (p.W) {      // the router's own products: eight entries at a time, every lane a share of the columns, fp32 throughout
+        const float* h = p.h + t * p.ldh;
+        const uint16_t* W = (const uint16_t*)p.W;
+        const int K = p.K;
+        const bool vec = (K & 3) == 0 && (p.ldh & 3) == 0 && ((uintptr_t)p.h & 15) == 0 && ((uintptr_t)p.W & 7) == 0;
+        for (int e0 = 0; e0 < E; e0 += 8) {
+            float acc[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+            if (vec) {
+                for (int k = lane * 4; k < K; k += 256) {
+                    const float4 x = *(const float4*)(h + k);
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        if (e0 + j < E) {
+                            const uint2 w = *(const uint2*)(W + (int64_t)(e0 + j) * K + k);
+                            acc[j] = fmaf(x.x, __uint_as_float(w.x << 16), acc[j]);
+                            acc[j] = fmaf(x.y, __uint_as_float(w.x & 0xffff0000u), acc[j]);
+                            acc[j] = fmaf(x.z, __uint_as_float(w.y << 16), acc[j]);
+                            acc[j] = fmaf(x.w, __uint_as_float(w.y & 0xffff0000u), acc[j]);
+                        }
+                    }
+                }
+            } else {
+                for (int k = lane; k < K; k += 64) {
+                    const float x = h[k];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        if (e0 + j < E) acc[j] = fmaf(x, __uint_as_float((uint32_t)W[(int64_t)(e0 + j) * K + k] << 16), acc[j]);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float v = wave_sum(acc[j]);
+                if (lane == 0 && e0 + j < E) ch[e0 + j] = v;
+            }
+        }
+    } else {
+        const float* z = p.logits + t * p.ld;
+        for (int e = lane; e < E; e += 64) ch[e] = z[e];
+    }
     float mx = -INFINITY;
-    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
+    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, ch[e]);
     mx = wave_max(mx);
     float sum = 0.0f;
     for (int e = lane; e < E; e += 64) {
-        const float v = expf(z[e] - mx);
+        const float v = expf(ch[e] - mx);
         sc[e] = v;
         sum += v;
     }
@@ -334,7 +372,7 @@ int i64h_route_topk(const i64h_route_args* dp, void* stream) {
     I64H_CHECK_ARG(d.E > 0 && d.E <= 1024 && d.top > 0 && d.top <= RT_MAX_TOP && d.top <= d.E, "route_topk: %d entries (at most 1024), top %d (at most %d)", d.E, d.top, RT_MAX_TOP);
     I64H_CHECK_ARG(d.groups <= 1 || (d.E % d.groups == 0 && d.keep >= 1 && d.keep <= d.groups), "route_topk: %d entries in %d groups, %d kept", d.E, d.groups, d.keep);
     I64H_CHECK_ARG(d.groups <= 1 || d.keep * (d.E / d.groups) >= d.top, "route_topk: %d kept groups of %d entries hold fewer than top %d", d.keep, d.E / (d.groups > 0 ? d.groups : 1), d.top);
-    I64H_CHECK_ARG(d.logits && d.idx && d.wgt && d.ld >= d.E, "route_topk: null operand or row stride below the entries");
+    I64H_CHECK_ARG(d.idx && d.wgt && ((d.logits && d.ld >= d.E) || (d.W && d.h && d.K > 0 && d.ldh >= d.K)), "route_topk: null operand or row stride below the row");
     if (d.n == 0) return 0;
     const size_t lds = 4 * (size_t)(2 * d.E + (d.groups > 1 ? d.groups : 1)) * 4;
     hipLaunchKernelGGL(route_topk_kernel, dim3((unsigned)((d.n + 3) / 4)), dim3(256), lds, (hipStream_t)stream, d);

@@ -410,19 +410,32 @@ def gla_scan(p: torch.Tensor, *, q_off: int, f_off: int, v_off: int, heads: int,
     return out
 
 
-def route_topk(logits: torch.Tensor, *, entries: int, correction: Optional[torch.Tensor], groups: int, keep: int, top: int, scale: float, idx: torch.Tensor,
-               wgt: torch.Tensor, n: Optional[int] = None) -> None:
-    """See i64h_route_topk.  logits fp32 [n, ld >= entries]; idx int32 [n, top]; wgt fp32 [n, top]."""
-    _chk(logits, torch.float32, "logits"), _chk(idx, torch.int32, "idx"), _chk(wgt, torch.float32, "wgt")
-    rows = int(n if n is not None else logits.shape[0])
+def route_topk(logits: Optional[torch.Tensor], *, entries: int, correction: Optional[torch.Tensor], groups: int, keep: int, top: int, scale: float, idx: torch.Tensor,
+               wgt: torch.Tensor, n: Optional[int] = None, h: Optional[torch.Tensor] = None, w: Optional[torch.Tensor] = None) -> None:
+    """See i64h_route_topk.  logits fp32 [n, ld >= entries], or None with h fp32 [n, K] and w bf16 [entries, K]: the launch computes the
+    logits itself in 32 bits; idx int32 [n, top]; wgt fp32 [n, top]."""
+    _chk(idx, torch.int32, "idx"), _chk(wgt, torch.float32, "wgt")
+    if logits is None:
+        if h is None or w is None:
+            raise _lib.I64HError("route_topk: logits, or the router's input and weight")
+        _chk(h, torch.float32, "h"), _chk(w, torch.bfloat16, "w")
+        rows = int(n if n is not None else h.shape[0])
+        if w.dim() != 2 or w.shape[0] != entries or h.shape[-1] != w.shape[1] or h.numel() < rows * h.shape[-1]:
+            raise _lib.I64HError("route_topk: the router's input and weight do not fit the sizes")
+    else:
+        _chk(logits, torch.float32, "logits")
+        rows = int(n if n is not None else logits.shape[0])
+        if logits.shape[-1] < entries or logits.numel() < rows * logits.shape[-1]:
+            raise _lib.I64HError("route_topk: shapes do not fit the sizes")
     if correction is not None:
         _chk(correction, torch.float32, "correction")
         if correction.numel() != entries:
             raise _lib.I64HError("route_topk: the correction is not [entries]")
-    if logits.shape[-1] < entries or logits.numel() < rows * logits.shape[-1] or idx.numel() < rows * top or wgt.numel() < rows * top:
+    if idx.numel() < rows * top or wgt.numel() < rows * top:
         raise _lib.I64HError("route_topk: shapes do not fit the sizes")
-    d = _lib.Route(logits=ptr(logits), ld=logits.shape[-1], E=entries, correction=ptr(correction), groups=int(groups), keep=int(keep), top=int(top),
-                   scale=float(scale), idx=ptr(idx), wgt=ptr(wgt), n=rows)
+    d = _lib.Route(logits=ptr(logits), ld=logits.shape[-1] if logits is not None else 0, E=entries, correction=ptr(correction), groups=int(groups), keep=int(keep),
+                   top=int(top), scale=float(scale), idx=ptr(idx), wgt=ptr(wgt), n=rows, h=ptr(h) if logits is None else 0,
+                   ldh=h.shape[-1] if logits is None else 0, W=ptr(w) if logits is None else 0, K=w.shape[1] if logits is None else 0)
     call_dense("i64h_route_topk", _ref(d), _stream())
 
 

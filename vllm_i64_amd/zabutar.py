@@ -114,7 +114,7 @@ class ZabutarModel:
         self.max_experts = max([m.experts for m in moes] or [0])
         self.max_shared = max([m.shared_ff for m in moes] or [0])
         self.max_act = max([l.mlp.ff for l in cfg.layers if l.mlp is not None and l.mlp.kind == "dense"] + [m.ff * m.top for m in moes] +
-                           [m.entries for m in moes] + [0])
+                           [0])
         if cache_dtype is None:
             cache_dtype = torch.float32 if self.exact else torch.bfloat16
         self.kv = HybridCache(specs, num_kv_blocks, max_seqs, dev, dtype=cache_dtype, block=kv_block, position_limit=cfg.max_positions)
@@ -271,9 +271,9 @@ class ZabutarModel:
     def _moe_ff(self, B, d, n, record=None, l=0) -> None:
         f, ex, W = d["mlp"], self.exact, self.cfg.width
         E, top = f.experts, f.top
-        logits = B.act[: n * f.entries].view(n, f.entries)
-        D.linear(B.hc, d["router"], logits, exact=True)      # the router's products in 32 bits in both modes: a choice is not rounding's to make
-        D.route_topk(logits, entries=f.entries, correction=d["correction"], groups=f.groups, keep=f.keep, top=top, scale=f.scale, idx=B.idx, wgt=B.wgt, n=n)
+        # the router's products in 32 bits in both modes (a choice between experts is not rounding's to make), inside the choice's launch
+        D.route_topk(None, h=B.hc, w=d["router"], entries=f.entries, correction=d["correction"], groups=f.groups, keep=f.keep, top=top, scale=f.scale,
+                     idx=B.idx, wgt=B.wgt, n=n)
         if record is not None:
             record[f"l{l}.route"] = B.idx[: n * top].view(n, top).clone()
         D.moe_plan(B.idx, n=n, top=top, experts=E, group_off=B.group_off, pair_token=B.pair_token, pair_row=B.pair_row)
