@@ -47,6 +47,17 @@ def test_registry_names_the_design():
     assert registry.architecture_of(config_of("plain")) == "Zabutar"
 
 
+def test_loader_takes_missing_sizes_from_the_tensors(monkeypatch):
+    from vllm_i64_amd import registry, zabutar
+    seen = {}
+    monkeypatch.setattr(zabutar, "ZabutarModel", lambda cfg, tensors, **kw: seen.setdefault("cfg", cfg))
+    d = config_of("odd")
+    for key in ("vocab", "width", "max_positions", "canon"):
+        d.pop(key)
+    cfg = registry._load_zabutar(d, make_weights("odd"), device="cpu", dtype="float32", max_seqs=2, max_tokens=64)
+    assert (cfg.vocab, cfg.width, cfg.max_positions, cfg.canon_taps) == (83, 40, 300, 3)
+
+
 def test_cache_shares_rows_between_layers_and_bounds_positions():
     from vllm_i64_amd.paged_cache import HybridCache
     kv = HybridCache([{"rows": 12, "kscale": False, "state": {"canon1": (2, 8)}}, {"state": {"gla": (2, 3, 4)}}, {"rows_of": 0, "state": {"canon1": (2, 8)}}],

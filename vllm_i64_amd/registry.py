@@ -47,6 +47,13 @@ def _load_dogalorn(config: dict, tensors, *, device, dtype, max_seqs, max_tokens
 def _load_zabutar(config: dict, tensors, *, device, dtype, max_seqs, max_tokens, kv_block=16, **_):
     from .config import ZabutarConfig
     from .zabutar import ZabutarModel
+    config = dict(config)
+    # sizes that the file may leave to the tensors' shapes
+    for key, name, axis in (("vocab", "embed", 0), ("width", "embed", 1), ("max_positions", "pos", 0)):
+        if key not in config and name in tensors:
+            config[key] = int(tensors[name].shape[axis])
+    if "canon" not in config and "l0.canon1" in tensors:
+        config["canon"] = {"taps": int(tensors["l0.canon1"].shape[1])}
     cfg = ZabutarConfig.from_dict(config)
     blocks = max(1, (int(max_tokens) + kv_block - 1) // kv_block)
     return ZabutarModel(cfg, tensors, device=device, dtype=dtype, max_seqs=max_seqs, num_kv_blocks=blocks, kv_block=kv_block)
