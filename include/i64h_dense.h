@@ -1,7 +1,10 @@
 /* libi64hip_dense.so - C ABI of the gfx950 (MI355X) kernels for decoder models with bf16 weights and a 32-bit residual:
  * tiled Linear on the bf16 / f32 matrix cores with fused epilogues, scaled embedding, gated post-norm residual with
  * grouped RMS norm and depth mixing, latent (low-rank, shared-key) attention over a paged cache with a sliding window,
- * row sampling.  A library of its own so that a process that serves such a model builds and loads nothing else.
+ * multi-stream and sandwich-norm residuals, causal convolutions with carried inputs, state-space / gated / gated-linear recurrences,
+ * attention with a distance bias (keys as values, or separate keys and values in one cached row), expert routing with grouped
+ * Linears over device-side row groups, row sampling.  A library of its own so that a process that serves such a model builds and
+ * loads nothing else.
  *
  * Conventions are those of libi64hip.so (include/i64h.h): raw device pointers, caller-allocated outputs, no allocation
  * and no synchronisation inside, 0 on success, the reason of a failure in i64h_last_error() of THIS library.

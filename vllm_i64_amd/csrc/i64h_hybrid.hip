@@ -1,13 +1,17 @@
 // Kernels of libi64hip_dense.so for recurrent and hybrid layers (include/i64h_dense.h, "recurrent and hybrid layers"):
 //   embed_bigram_kernel / prev_token_kernel : token embedding + hashed bigram embedding; the previous token is per-sequence state
-//   streams_kernel        : multi-stream residual write + the next sublayer's weighted read and RMS norm, one workgroup per row
-//   causal_conv_kernel / conv_carry_kernel : per-channel causal convolution + silu over rows and carried inputs; the carry update
+//   streams_kernel        : multi-stream residual write (a result may pass a norm of its own first) + the next sublayer's weighted read
+//                           and RMS norm, one workgroup per row
+//   causal_conv_kernel / conv_carry_kernel : per-channel causal convolution over rows and carried inputs (+ silu, or added to its input);
+//                           the carry update
 //   ssm_scan_kernel       : state-space recurrence with a scalar decay per head, a head's matrix in registers (16 lanes per value column)
 //   gate_norm_kernel      : y * silu(z) -> RMS norm in groups
 //   mingru_scan_kernel    : element-wise gated recurrence, tiles of 64 tokens scanned by four waves and folded
 //   kattn_prep_kernel     : whole-row RMS norms of query and key, key-norm weights / scale / temperature folded into the query,
 //                           raw key row and its 1 / rms into the paged cache
-//   kattn_row_kernel      : attention over the cached keys (which are also the values) with distance bias, chunk mask and sink
+//   kattn_row_kernel      : attention over the cached keys (which are also the values, or with the values in front of them in the
+//                           same cached row) with distance bias, chunk mask and sink
+//   kv_prep_kernel        : [q | k | v] projections -> the cached row [v | k] per key head and query rows with zeros in the value columns
 // A row continues the row before it iff slot and position say so; state is taken as empty at position 0.  All arithmetic fp32.
 #include "i64h_common.h"
 #include "i64h_dense.h"
