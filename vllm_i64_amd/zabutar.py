@@ -295,9 +295,9 @@ class ZabutarModel:
         """token_ids int64 [N]; positions / slot_ids int32 [N], rows in sequence order (the rows of a sequence consecutive, positions
         consecutive, continuing what the sequence's slot and pages hold; position 0 starts a sequence afresh); logit_rows int32 [M]
         selects the rows whose logits are wanted (None = all).  Returns fp32 logits [M, V].  record: dict filled with the residual after
-        every layer ("l<i>.x") and every mixture layer's chosen entries ("l<i>.route", int32 [N, top]).  kv: a HybridCache other than the runner's own.  tokens_per_seq (rows per sequence, in order) or
-        rows_are_slots (every row a sequence of its own) say how the rows are grouped; without them the slot ids are read back.
-        ctx_len and max_ctx_hint belong to the shared step interface."""
+        every layer ("l<i>.x") and every mixture layer's chosen entries ("l<i>.route", int32 [N, top]).  kv: a HybridCache other than the
+        runner's own.  tokens_per_seq (rows per sequence, in order) or rows_are_slots (every row a sequence of its own) say how the rows
+        are grouped; without them the slot ids are read back.  ctx_len and max_ctx_hint belong to the shared step interface."""
         cfg = self.cfg
         kvc = kv if kv is not None else self.kv
         n = token_ids.numel()
