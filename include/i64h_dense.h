@@ -33,6 +33,7 @@ int i64h_device_check(void);
  *   I64H_EPI_SOFTCAP: cap * tanh(. / cap);  I64H_EPI_GELU_ERF: 0.5 v (1 + erf(v / sqrt 2));  I64H_EPI_SCALE: v * scale;
  *   I64H_EPI_SILU_MUL: silu(A W^T) * (A W2^T), laid out as I64H_EPI_GELU_MUL;
  *   I64H_EPI_XIELU: v > 0 ? act_a v^2 + v / 2 : act_b (exp(v) - 1 - v) + v / 2  (the caller passes act_a = softplus(p), act_b = 1/2 + softplus(q)).
+ *   I64H_EPI_RELU_SQ: max(v, 0)^2.
  *   bias (may be NULL; fp32 [N], batch stride bias_batch) is added to the sum before any epilogue but the two gate / up ones.
  * group_off (may be NULL; device int32 [batch + 1], ascending): batch b takes the rows [group_off[b], group_off[b + 1]) of a_rows
  *   (of A itself without a_rows) and of C instead of all M rows; M is then the most rows any batch may have (it sizes the launch,
@@ -48,6 +49,7 @@ int i64h_device_check(void);
 #define I64H_EPI_SCALE 5
 #define I64H_EPI_SILU_MUL 6
 #define I64H_EPI_XIELU 7
+#define I64H_EPI_RELU_SQ 8
 #define I64H_SKINNY_ROWS 8
 typedef struct {
     const float* A;
@@ -138,7 +140,8 @@ int i64h_latent_prep(const i64h_latent_prep_args* d, void* stream);
 /* i64h_latent_attn: row t (sequence slot_ids[t], position p = positions[t]) sees the cached rows j of its sequence with
  * 0 <= p - j < window (window <= 0: every j <= p);  s_j = scale * Q[t, h, :] . row_j;  ordinary softmax over the visible j;
  * out[t, h, :kv_rank] = sum_j w_j * row_j[:kv_rank].  Scores, weights and sums in fp32.  out fp32 [n, heads, kv_rank].
- * mode 1: one wave per (row, head), fp32 products, any sizes and cache type.  Modes 0 / 2 / 3 take the matrix-core form when the cache
+ * With sink the denominator also holds exp(sink_w[h]) (exp(0) without sink_w): a term without a key and without a value, not scaled.
+ * mode 1: one wave per (row, head), fp32 products, any sizes and cache type (of the options below it knows the sink).  Modes 0 / 2 / 3 take the matrix-core form when the cache
  * is bf16, kv_rank % 16 == 0 and <= 256, (kv_rank + rot_dim) % 8 == 0 and <= 320 (the row form otherwise): 2 (and 0) one wave per token
  * and group of 16 heads (rows that are one per sequence), 3 one wave per 16 consecutive rows and head (portions of prompts; rows of
  * different sequences in one tile are handled run by run). */
@@ -168,6 +171,8 @@ typedef struct {
     int32_t sink;        /* one more score of zero, without a value, in the softmax's denominator */
     int32_t key_off;     /* the first key_off columns of a cached row part carry values only: the caller's query is zero there, and the score
                             products over 32-column steps that lie wholly inside them are left out */
+    const float* sink_w; /* with sink: fp32 [heads], the extra score of head h is sink_w[h] instead of zero (NULL: zero) */
+    float softcap;       /* > 0: a score s (after scale and key scale, before any bias) becomes softcap * tanh(s / softcap) */
 } i64h_latent_attn_args;
 int i64h_set_latent_attn_decode_form(int32_t on); /* tuning / test knob: 1 (default) = mode 2 launches run the kernel that requests a tile's fragments a tile ahead; 0 = the general matrix-core kernel; same results up to summation order */
 int64_t i64h_latent_attn_workspace_floats(int64_t n, int32_t heads, int32_t kv_rank, int32_t splits);
@@ -180,7 +185,7 @@ int i64h_latent_attn(const i64h_latent_attn_args* d, void* stream);
  * clearing).  seg_start [nseg + 1] lists the first row of every run of consecutive rows of one sequence (seg_start[nseg] = n). */
 
 /* ---- token embedding + hashed bigram embedding ----------------------------------------------------------------------------------
- * out[c][t, :] = table[ids[t]] + bigram[row(t)] for c < copies (out fp32 [copies, n, W]);  row(t) = buckets at position 0, else
+ * out[c][t, :] = table[ids[t]] * scale + bigram[row(t)] for c < copies (out fp32 [copies, n, W]);  row(t) = buckets at position 0, else
  * (previous * mul_prev + ids[t] * mul_cur) mod buckets, previous = the token of the row before in the same sequence, or
  * prev_token[slot] (the last token of the sequence's earlier steps).  A second launch stores every sequence's last token of
  * this step in prev_token.  bigram == NULL: the token embedding alone.  pos_table (may be NULL; bf16 [pos_rows, W]): the row of the
@@ -200,6 +205,7 @@ typedef struct {
     int64_t n;
     const void* pos_table;
     int64_t pos_rows;
+    float scale;         /* multiplies the token row only (not the bigram or position rows) */
 } i64h_embed_bigram_args;
 int i64h_embed_bigram(const i64h_embed_bigram_args* d, void* stream);
 
@@ -207,8 +213,11 @@ int i64h_embed_bigram(const i64h_embed_bigram_args* d, void* stream);
  * streams fp32 [S, n, W], updated in place, one workgroup per row:
  *   write (y != NULL):  v = y2 ? 0.5 * (rms(y) * yn_w + rms(y2) * y2n_w) : (yn_w ? rms(y) * yn_w : y)
  *                       (rms over the W columns with y_eps; weights [W]; a single normed result is the post-norm of a sandwich layer)
+ *                       post_w != NULL: v <- norm(v) * post_w, over the W columns with y_eps - the root mean square, or with post_center the
+ *                       centred norm (v - mean) / sqrt(mean((v - mean)^2) + y_eps): a norm on a sublayer's result, whatever it is made of
  *                       new_t = sum_s mix[s * S + t] * old_s + out_w[t] * v          (mix == NULL: new_t = old_t + out_w[t] * v)
- *   read  (h != NULL):  u = sum_s in_w[s] * x_s  (in_w == NULL: the plain sum);  h = u / sqrt(mean(u^2) + eps) * norm_w[c % norm_w_len]
+ *   read  (h != NULL):  u = sum_s in_w[s] * x_s  (in_w == NULL: the plain sum);  h = u / sqrt(mean(u^2) + eps) * norm_w[c % norm_w_len],
+ *                       or with h_center the centred norm (u - mean) / sqrt(mean((u - mean)^2) + eps) * norm_w
  * rows (may be NULL, read only launches): h[m] is computed from row rows[m] of the streams (the rows whose logits are wanted). */
 typedef struct {
     float* streams;
@@ -231,6 +240,9 @@ typedef struct {
     float* h;
     const int32_t* rows;
     int64_t m_rows;
+    const float* post_w;
+    int32_t post_center;
+    int32_t h_center;
 } i64h_streams_args;
 int i64h_streams_step(const i64h_streams_args* d, void* stream);
 
@@ -285,7 +297,8 @@ typedef struct {
 int i64h_ssm_scan(const i64h_ssm_scan_args* d, void* stream);
 
 /* out[t, :] = rms_groups(y[t, :] * silu(z[t, :])) * w: the `width` columns in `groups` equal consecutive parts, each divided by
- * sqrt(mean(part^2) + eps).  z == NULL: no gate. */
+ * sqrt(mean(part^2) + eps).  z == NULL: no gate.  gate_after: out = rms_groups(y) * w * silu(z), the gate behind the norm.
+ * w_len (0: width) values of w, repeated over the columns (a head norm whose weights all heads share). */
 typedef struct {
     const float* y;
     int64_t ldy;
@@ -297,6 +310,8 @@ typedef struct {
     float* out;
     int64_t ldo;
     int64_t n;
+    int32_t gate_after;
+    int32_t w_len;
 } i64h_gate_norm_args;
 int i64h_gate_norm(const i64h_gate_norm_args* d, void* stream);
 
@@ -376,6 +391,7 @@ typedef struct {
     int32_t vdim;        /* > 0: keys and values are separate (see i64h_kv_prep): a cached row holds per key head [vdim values | dim key values], Q is
                             [n, heads, vdim + dim] with the query in the last dim columns of a head, out [n, heads, vdim], kscale may be NULL;
                             the workspace is then i64h_kattn_workspace_floats(n, heads, kv_heads, vdim, splits) floats */
+    float softcap;       /* > 0: the score Q . k * kscale becomes softcap * tanh(. / softcap) before the bias is added */
 } i64h_kattn_args;
 int64_t i64h_kattn_workspace_floats(int64_t n, int32_t heads, int32_t kv_heads, int32_t dim, int32_t splits);
 int i64h_kattn(const i64h_kattn_args* d, void* stream);
@@ -426,6 +442,83 @@ typedef struct {
 } i64h_gla_args;
 int i64h_gla_gates(const i64h_gla_args* d, void* stream);
 int i64h_gla_scan(const i64h_gla_args* d, void* stream);
+
+/* ---- attention with rotated queries, keys and (optionally) values over [values | keys] rows ---------------------------------------------
+ * i64h_rot_prep, per row t of the projections P (position pos):  q = P[t, q_off : + heads * dim], k = P[t, k_off : + kv_heads * dim],
+ * v = P[t, v_off : + kv_heads * vdim];
+ *   1. q_norm_w / k_norm_w (may be NULL, together): q <- q / sqrt(mean(q^2) + eps) * q_norm_w over the WHOLE row of heads * dim values, k likewise;
+ *   2. the first rot_dims values of every head turn by pos * inv_freq[i] (fp32 product, full-range sine / cosine, both multiplied by rot_mult):
+ *      pairs (i, i + rot_dims / 2) or, with interleaved, (2i, 2i + 1); (u, v) -> (u cos - v sin, v cos + u sin); the rest pass unchanged;
+ *   3. head_norm: q and k are divided by sqrt(mean over the head's dim values of the square + eps), no weight;
+ *   4. v_freq (may be NULL; fp32 [vdim / 2]): all vdim values of every value head turn by pos * v_freq[m], pairs in the same layout;
+ *   cache row (slot, position) <- per key head g: [v_g (vdim) | k_g (dim)];   Q[t, h, :] = [0 (vdim) | q_h * scale (dim)].
+ * i64h_kattn (vdim > 0) on these computes the attention; i64h_rot_post finishes its output in place:
+ *   O[t, h, :] turns by -pos * v_freq[m] (v_freq may be NULL: no turn) and is multiplied by sigmoid(gate[t, h]) (gate may be NULL; row stride ldg). */
+typedef struct {
+    const float* P;
+    int64_t ldp;
+    int32_t q_off, k_off, v_off;
+    int32_t heads, kv_heads, dim, vdim;
+    const float* q_norm_w;
+    const float* k_norm_w;
+    float eps;
+    int32_t rot_dims, interleaved;
+    const float* inv_freq;
+    float rot_mult;
+    int32_t head_norm;
+    const float* v_freq;
+    float scale;
+    const int32_t* positions;
+    const int32_t* slot_ids;
+    const int32_t* block_table;
+    int32_t max_blocks_per_seq, block_size;
+    void* cache;
+    int32_t cache_dtype;
+    float* Q;
+    int64_t n;
+} i64h_rot_prep_args;
+int i64h_rot_prep(const i64h_rot_prep_args* d, void* stream);
+typedef struct {
+    float* O;            /* fp32 [n, heads, vdim], in place */
+    int32_t heads, vdim, interleaved;
+    const float* v_freq;
+    const int32_t* positions;
+    const float* gate;
+    int64_t ldg;
+    int64_t n;
+} i64h_rot_post_args;
+int i64h_rot_post(const i64h_rot_post_args* d, void* stream);
+
+/* ---- gated delta rule -------------------------------------------------------------------------------------------------------------------
+ * Per sequence and head a (dim x vdim) matrix S in fp32, head a reading the query / key head a / (heads / kv_heads):
+ *   S <- g_t S;   u = beta_t (v_t - S^T k_t);   S <- S + k_t u^T;   o_t = S^T q_t       (the read-out sees the token's own write)
+ * q_t = X[t, q_off + j * dim : + dim], k_t likewise at k_off, v_t = X[t, v_off + a * vdim : + vdim]; beta_t = G[t, a], g_t = G[t, heads + a].
+ * i64h_gdn_gates prepares them: q and k of every query / key head divided by sqrt(sum of squares + unit_eps) in place (unit_eps < 0: left as
+ * they are), q times q_scale;  G[t, a] = sigmoid(R[t, b_off + a]),  G[t, heads + a] = exp(-exp(A_log[a]) * softplus(R[t, a_off + a] + dt_bias[a])).
+ * state fp32 [slots, heads, vdim, dim] (S transposed; dim <= 256).  All arithmetic fp32, the tokens of a sequence strictly in their order. */
+typedef struct {
+    float* X;
+    int64_t ldx;
+    int32_t q_off, k_off, v_off;
+    int32_t heads, kv_heads, dim, vdim;
+    float* G;            /* fp32 [n, 2 * heads] */
+    const float* R;      /* raw projections of beta and of the decay's step (gates only) */
+    int64_t ldr;
+    int32_t b_off, a_off;
+    const float* A_log;
+    const float* dt_bias;
+    float unit_eps, q_scale;
+    const int32_t* seg_start;
+    int32_t nseg;
+    const int32_t* positions;
+    const int32_t* slot_ids;
+    float* state;
+    float* out;          /* fp32 [n, heads * vdim], row stride ldo */
+    int64_t ldo;
+    int64_t n;
+} i64h_gdn_args;
+int i64h_gdn_gates(const i64h_gdn_args* d, void* stream);
+int i64h_gdn_scan(const i64h_gdn_args* d, void* stream);
 
 /* ---- router: softmax scores, corrected choice, groups of neighbours, top-k ---------------------------------------------------------------------
  * Per row t of logits (fp32, row stride ld, E entries):  s = softmax(logits[t]);  choice = s + correction (correction may be NULL);

@@ -224,6 +224,10 @@ DENSE_SIGNATURES: Dict[str, str] = {
     "i64h_kattn_prep": "pp",
     "i64h_kattn": "pp",
     "i64h_kv_prep": "pp",
+    "i64h_rot_prep": "pp",
+    "i64h_rot_post": "pp",
+    "i64h_gdn_gates": "pp",
+    "i64h_gdn_scan": "pp",
     "i64h_gla_gates": "pp",
     "i64h_gla_scan": "pp",
     "i64h_route_topk": "pp",
@@ -258,20 +262,20 @@ class LatentAttn(ctypes.Structure):
     _fields_ = [("Q", _P), ("cache", _P), ("cache_dtype", _I), ("block_table", _P), ("max_blocks_per_seq", _I), ("block_size", _I),
                 ("slot_ids", _P), ("positions", _P), ("window", _I), ("scale", _F), ("out", _P), ("n", _L), ("heads", _I), ("kv_rank", _I),
                 ("rot_dim", _I), ("mode", _I), ("splits", _I), ("workspace", _P), ("row_stride", _I), ("kv_groups", _I), ("chunk", _I), ("kscale", _P),
-                ("bias", _P), ("bias_rows", _I), ("sink", _I), ("key_off", _I)]
+                ("bias", _P), ("bias_rows", _I), ("sink", _I), ("key_off", _I), ("sink_w", _P), ("softcap", _F)]
 
 
 class EmbedBigram(ctypes.Structure):
     """Mirror of i64h_embed_bigram_args (include/i64h_dense.h)."""
     _fields_ = [("ids", _P), ("positions", _P), ("slot_ids", _P), ("table", _P), ("V", _L), ("W", _I), ("bigram", _P), ("buckets", _L),
-                ("mul_prev", _L), ("mul_cur", _L), ("prev_token", _P), ("out", _P), ("copies", _I), ("n", _L), ("pos_table", _P), ("pos_rows", _L)]
+                ("mul_prev", _L), ("mul_cur", _L), ("prev_token", _P), ("out", _P), ("copies", _I), ("n", _L), ("pos_table", _P), ("pos_rows", _L), ("scale", _F)]
 
 
 class Streams(ctypes.Structure):
     """Mirror of i64h_streams_args (include/i64h_dense.h)."""
     _fields_ = [("streams", _P), ("S", _I), ("n", _L), ("W", _I), ("y", _P), ("ldy", _L), ("y2", _P), ("ldy2", _L), ("yn_w", _P), ("y2n_w", _P),
                 ("y_eps", _F), ("mix", _P), ("out_w", _P), ("in_w", _P), ("norm_w", _P), ("norm_w_len", _I), ("eps", _F), ("h", _P), ("rows", _P),
-                ("m_rows", _L)]
+                ("m_rows", _L), ("post_w", _P), ("post_center", _I), ("h_center", _I)]
 
 
 class CausalConv(ctypes.Structure):
@@ -289,7 +293,8 @@ class SsmScan(ctypes.Structure):
 
 class GateNorm(ctypes.Structure):
     """Mirror of i64h_gate_norm_args (include/i64h_dense.h)."""
-    _fields_ = [("y", _P), ("ldy", _L), ("z", _P), ("ldz", _L), ("w", _P), ("width", _I), ("groups", _I), ("eps", _F), ("out", _P), ("ldo", _L), ("n", _L)]
+    _fields_ = [("y", _P), ("ldy", _L), ("z", _P), ("ldz", _L), ("w", _P), ("width", _I), ("groups", _I), ("eps", _F), ("out", _P), ("ldo", _L), ("n", _L),
+                ("gate_after", _I), ("w_len", _I)]
 
 
 class MinGruScan(ctypes.Structure):
@@ -309,7 +314,7 @@ class KAttn(ctypes.Structure):
     """Mirror of i64h_kattn_args (include/i64h_dense.h)."""
     _fields_ = [("Q", _P), ("cache", _P), ("cache_dtype", _I), ("kscale", _P), ("block_table", _P), ("max_blocks_per_seq", _I), ("block_size", _I),
                 ("slot_ids", _P), ("positions", _P), ("chunk", _I), ("bias", _P), ("bias_rows", _I), ("sink", _I), ("out", _P), ("n", _L), ("heads", _I),
-                ("kv_heads", _I), ("dim", _I), ("mode", _I), ("splits", _I), ("workspace", _P), ("vdim", _I)]
+                ("kv_heads", _I), ("dim", _I), ("mode", _I), ("splits", _I), ("workspace", _P), ("vdim", _I), ("softcap", _F)]
 
 
 class KvPrep(ctypes.Structure):
@@ -317,6 +322,26 @@ class KvPrep(ctypes.Structure):
     _fields_ = [("P", _P), ("ldp", _L), ("q_off", _I), ("k_off", _I), ("v_off", _I), ("heads", _I), ("kv_heads", _I), ("dim", _I), ("vdim", _I),
                 ("scale", _F), ("positions", _P), ("slot_ids", _P), ("block_table", _P), ("max_blocks_per_seq", _I), ("block_size", _I),
                 ("cache", _P), ("cache_dtype", _I), ("Q", _P), ("n", _L)]
+
+
+class RotPrep(ctypes.Structure):
+    """Mirror of i64h_rot_prep_args (include/i64h_dense.h)."""
+    _fields_ = [("P", _P), ("ldp", _L), ("q_off", _I), ("k_off", _I), ("v_off", _I), ("heads", _I), ("kv_heads", _I), ("dim", _I), ("vdim", _I),
+                ("q_norm_w", _P), ("k_norm_w", _P), ("eps", _F), ("rot_dims", _I), ("interleaved", _I), ("inv_freq", _P), ("rot_mult", _F),
+                ("head_norm", _I), ("v_freq", _P), ("scale", _F), ("positions", _P), ("slot_ids", _P), ("block_table", _P),
+                ("max_blocks_per_seq", _I), ("block_size", _I), ("cache", _P), ("cache_dtype", _I), ("Q", _P), ("n", _L)]
+
+
+class RotPost(ctypes.Structure):
+    """Mirror of i64h_rot_post_args (include/i64h_dense.h)."""
+    _fields_ = [("O", _P), ("heads", _I), ("vdim", _I), ("interleaved", _I), ("v_freq", _P), ("positions", _P), ("gate", _P), ("ldg", _L), ("n", _L)]
+
+
+class Gdn(ctypes.Structure):
+    """Mirror of i64h_gdn_args (include/i64h_dense.h)."""
+    _fields_ = [("X", _P), ("ldx", _L), ("q_off", _I), ("k_off", _I), ("v_off", _I), ("heads", _I), ("kv_heads", _I), ("dim", _I), ("vdim", _I),
+                ("G", _P), ("R", _P), ("ldr", _L), ("b_off", _I), ("a_off", _I), ("A_log", _P), ("dt_bias", _P), ("unit_eps", _F), ("q_scale", _F),
+                ("seg_start", _P), ("nseg", _I), ("positions", _P), ("slot_ids", _P), ("state", _P), ("out", _P), ("ldo", _L), ("n", _L)]
 
 
 class Gla(ctypes.Structure):

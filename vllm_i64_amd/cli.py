@@ -30,7 +30,7 @@ def _load(args, max_seqs: int, max_tokens: int):
     from .registry import architecture_of, load_model
     with open(os.path.join(args.model, "config.json"), "r", encoding="utf-8") as f:
         config = json.load(f)
-    _ensure_built(dense_only=architecture_of(config).lower() in ("morilorn", "dogalorn", "zabutar"))
+    _ensure_built(dense_only=architecture_of(config).lower() in ("morilorn", "dogalorn", "zabutar", "fukatar"))
     if not torch.cuda.is_available():
         raise SystemExit("no GPU: this package has no CPU path")
     return load_model(args.model, dtype=args.dtype, device="cuda:0", max_seqs=max_seqs, max_tokens=max_tokens, config=config)

@@ -89,6 +89,7 @@ class LatentAttentionConfig:
     window: int = 0          # a position sees itself and the window - 1 before it; 0: all earlier positions
     rot_base: float = 10000.0
     rot_dims: int = 0        # leading dimensions of the rotated part that are rotated (the rest pass through)
+    sink: bool = False       # a learned score per head in the softmax's denominator, without key or value (tensor 'sink')
 
     @property
     def q_width(self) -> int:
@@ -99,13 +100,13 @@ class LatentAttentionConfig:
         return self.kv_rank + self.rot_dim
 
     @classmethod
-    def from_dict(cls, m: dict) -> "LatentAttentionConfig":
+    def from_dict(cls, m: dict, sink: bool = False) -> "LatentAttentionConfig":
         rot = m.get("rot") or {}
         rot_dim = int(m.get("rot_dim", 0))
         mask = m.get("mask") or {}
         c = cls(heads=int(m["heads"]), dim=int(m["dim"]), rot_dim=rot_dim, vdim=int(m["vdim"]), kv_rank=int(m["kv_rank"]),
                 scale=float(m["scale"]), window=int(mask.get("size", 0)), rot_base=float(rot.get("base", 10000.0)),
-                rot_dims=int(rot.get("dims", rot_dim)) if rot_dim else 0)
+                rot_dims=int(rot.get("dims", rot_dim)) if rot_dim else 0, sink=bool(sink))
         if c.rot_dims > c.rot_dim or c.rot_dims % 2:
             raise ValueError(f"latent_attention: {c.rot_dims} rotated dimensions do not fit a rotated part of {c.rot_dim}")
         if min(c.heads, c.dim, c.vdim, c.kv_rank) <= 0 or c.window < 0:
@@ -323,7 +324,9 @@ class DecoderLayerConfig:
     weights_of: "int | None" = None      # the layer whose tensors this layer uses (its cache and state stay its own)
 
     @classmethod
-    def from_dict(cls, d: dict) -> "DecoderLayerConfig":
+    def from_dict(cls, d: dict, mixers: "dict | None" = None) -> "DecoderLayerConfig":
+        """mixers: a design's own table of layer type -> reader of the 'mixer' entry, where its types mean other mixers than MIXERS'."""
+        MIXERS = mixers if mixers is not None else globals()["MIXERS"]
         kind = d.get("type")
         if kind not in MIXERS:
             raise ValueError(f"layer type '{kind}' is not built (known: {sorted(MIXERS)})")
@@ -331,7 +334,8 @@ class DecoderLayerConfig:
         share = d.get("weights_of")
         if mlp and mlp.get("kind", "dense") not in MLPS:
             raise ValueError(f"feed-forward kind '{mlp.get('kind')}' is not built (known: {sorted(MLPS)})")
-        return cls(type=kind, mixer=MIXERS[kind].from_dict(d["mixer"]), mlp=MLPS[mlp.get("kind", "dense")].from_dict(mlp) if mlp else None,
+        reader = MIXERS[kind]
+        return cls(type=kind, mixer=reader.from_dict(d["mixer"]) if hasattr(reader, "from_dict") else reader(d["mixer"]), mlp=MLPS[mlp.get("kind", "dense")].from_dict(mlp) if mlp else None,
                    weights_of=int(share) if share is not None else None)
 
 
@@ -513,3 +517,190 @@ class ZabutarConfig:
         return {"architecture": "Zabutar", "vocab": self.vocab, "width": self.width, "max_positions": self.max_positions, "norm": {"eps": self.norm_eps},
                 "canon": {"taps": self.canon_taps},
                 "layers": [{"type": l.type, "mixer": l.mixer.to_dict(), "mlp": l.mlp.to_dict() if l.mlp else None} for l in self.layers]}
+
+
+# ---------------------------------------------------------------------------------------------------------------------------
+# Fukatar: a decoder whose sublayers read the residual itself and whose results pass a centred norm before they are added; the
+# mixer's input is first blended per channel with the row before (token shift); scaled embedding plus a hashed bigram row; per
+# layer one of three mixers: softmax attention with rotated queries, keys AND values (whole-row query / key norms, capped scores,
+# a sigmoid gate per head), latent attention without positions and with a learned sink, or a capped unit-norm attention side by
+# side with a gated delta rule; feed-forwards with a squared relu; capped logits.  Every size and constant comes from config.json.
+# ---------------------------------------------------------------------------------------------------------------------------
+@dataclass
+class RotaryConfig:
+    """Rotation of the first `dims` values of a head by position * base^(-2i / dims).  With scaling the frequencies whose period is
+    long against `original` positions are divided by `factor`, the short-period ones kept, with a linear ramp over the pair index
+    between the two at which `original` positions make `fast` and `slow` turns; sine and cosine then carry 0.1 ln(factor) + 1."""
+    base: float
+    dims: int
+    factor: float = 0.0          # 0: no scaling
+    original: float = 0.0
+    fast: float = 0.0
+    slow: float = 0.0
+
+    @classmethod
+    def from_dict(cls, r: dict) -> "RotaryConfig":
+        sc = r.get("scaling") or {}
+        c = cls(base=float(r["base"]), dims=int(r["dims"]), factor=float(sc.get("factor", 0.0)), original=float(sc.get("original", 0.0)),
+                fast=float(sc.get("fast", 0.0)), slow=float(sc.get("slow", 0.0)))
+        if c.dims < 0 or c.dims % 2 or c.base <= 1.0 or (c.factor and min(c.factor, c.original, c.fast, c.slow) <= 0):
+            raise ValueError(f"rotation: bad constants {r}")
+        return c
+
+    def to_dict(self) -> dict:
+        d = {"base": self.base, "dims": self.dims}
+        if self.factor:
+            d["scaling"] = {"factor": self.factor, "original": self.original, "fast": self.fast, "slow": self.slow}
+        return d
+
+    def frequencies(self):
+        """([dims / 2] frequencies evaluated in 64 bits, the factor on sine and cosine)."""
+        import math
+        half, D, b = self.dims // 2, self.dims, self.base
+        f = [b ** (-2.0 * i / D) for i in range(half)]
+        if not self.factor:
+            return f, 1.0
+        where = lambda turns: D * math.log(self.original / (2.0 * math.pi * turns)) / (2.0 * math.log(b))
+        lo, hi = max(math.floor(where(self.fast)), 0), min(math.ceil(where(self.slow)), D - 1)
+        for i in range(half):
+            ramp = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+            f[i] = f[i] / self.factor * ramp + f[i] * (1.0 - ramp)
+        return f, 0.1 * math.log(self.factor) + 1.0
+
+
+@dataclass
+class RotaryAttentionConfig:
+    """Causal softmax attention over grouped key / value heads with separate key and value sizes and rotated positions.  What a design
+    fixes comes in as flags: qk_norm 'row' (RMS norm over the whole projection with weights 'q.norm' / 'k.norm', before the rotation),
+    'head' (per head, without weights, after it) or None; interleaved pairs (2i, 2i + 1) or halves (i, i + dims / 2); rotated values
+    (all vdim dimensions by the value's own position, the head's sum turned back by the query's); a sigmoid gate per head ('g')."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    softcap: float = 0.0           # 0: scores are not capped
+    rot: "RotaryConfig | None" = None
+    qk_norm: "str | None" = None
+    interleaved: bool = False
+    rotate_values: bool = False
+    head_gate: bool = False
+
+    @classmethod
+    def from_dict(cls, m: dict, **design) -> "RotaryAttentionConfig":
+        c = cls(heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])), dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])), scale=float(m["scale"]),
+                softcap=float(m.get("softcap") or 0.0), rot=RotaryConfig.from_dict(m["rot"]) if m.get("rot") else None, **design)
+        if min(c.heads, c.kv_heads, c.dim, c.vdim) <= 0 or c.heads % c.kv_heads or c.softcap < 0 or (c.rot is not None and c.rot.dims > c.dim):
+            raise ValueError(f"attention: bad sizes {m}")
+        if c.rotate_values and c.rot is not None and c.vdim % 2:
+            raise ValueError(f"attention: rotated values of an odd size {c.vdim}")
+        return c
+
+    def to_dict(self) -> dict:
+        d = {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim, "scale": self.scale}
+        if self.softcap:
+            d["softcap"] = self.softcap
+        if self.rot is not None:
+            d["rot"] = self.rot.to_dict()
+        return d
+
+
+@dataclass
+class GatedDeltaConfig:
+    """Gated delta rule: per head a (dim x vdim) matrix that decays by a scalar per head and token, is corrected towards the value along
+    the (unit) key with a sigmoid strength, and is read by the (unit, scaled) query after the write; `kv_heads` query / key heads serve
+    `heads` value heads; a causal convolution of `conv` taps and silu in front of q, k and v; a gated RMS norm over vdim behind."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    conv: int = 1
+
+    @property
+    def conv_channels(self) -> int:
+        return 2 * self.kv_heads * self.dim + self.heads * self.vdim
+
+    @classmethod
+    def from_dict(cls, m: dict) -> "GatedDeltaConfig":
+        c = cls(heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])), dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])), conv=int(m.get("conv", 1)))
+        if min(c.heads, c.kv_heads, c.dim, c.vdim, c.conv) <= 0 or c.heads % c.kv_heads:
+            raise ValueError(f"gated delta rule: bad sizes {m}")
+        return c
+
+    def to_dict(self) -> dict:
+        return {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim, "conv": self.conv}
+
+
+def _fukatar_latent(m: dict) -> LatentAttentionConfig:
+    c = LatentAttentionConfig.from_dict(m, sink=True)
+    if c.rot_dim or c.window:
+        raise ValueError("latent attention of this design has no rotated part and no window")
+    return c
+
+
+def _fukatar_parallel(m: dict) -> ParallelMixerConfig:
+    return ParallelMixerConfig(left=RotaryAttentionConfig.from_dict(m["left"], qk_norm="head", interleaved=True),
+                               right=GatedDeltaConfig.from_dict(m["right"]))
+
+
+FUKATAR_MIXERS = {"attention": lambda m: RotaryAttentionConfig.from_dict(m, qk_norm="row", rotate_values=True, head_gate=True),
+                  "latent_attention": _fukatar_latent, "parallel": _fukatar_parallel}
+
+
+@dataclass
+class FukatarConfig:
+    vocab: int
+    width: int
+    layers: list
+    norm_eps: float = 1e-6
+    embedding_scale: float = 1.0
+    bigram: "BigramConfig | None" = None
+    logit_softcap: float = 0.0     # 0: logits are not capped
+    name: str = "Fukatar"
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def vocab_size(self) -> int:
+        return self.vocab
+
+    @property
+    def max_pos(self) -> int:
+        """Positions are computed, not tabulated: a sequence is bounded by the page pool only."""
+        return 1 << 30
+
+    @classmethod
+    def from_dict(cls, d: dict) -> "FukatarConfig":
+        emb = d.get("embedding") or {}
+        bg = emb.get("bigram")
+        layers = [DecoderLayerConfig.from_dict(l, FUKATAR_MIXERS) for l in d["layers"]]
+        c = cls(vocab=int(d["vocab"]), width=int(d["width"]), layers=layers, norm_eps=float((d.get("norm") or {}).get("eps", 1e-6)),
+                embedding_scale=float(emb.get("scale", 1.0)), bigram=BigramConfig(int(bg["buckets"]), int(bg["mul_prev"]), int(bg["mul_cur"])) if bg else None,
+                logit_softcap=float(d.get("logit_softcap") or 0.0), name=str(d.get("architecture", "Fukatar")))
+        if min(c.vocab, c.width) <= 0 or (c.bigram is not None and c.bigram.buckets <= 0):
+            raise ValueError("bad sizes")
+        for i, l in enumerate(layers):
+            if l.weights_of is not None:
+                raise ValueError(f"layer {i}: this design has no layers that borrow tensors")
+            if l.mlp is not None and l.mlp.kind != "dense":
+                raise ValueError(f"layer {i}: feed-forward kind '{l.mlp.kind}' is not part of this design")
+        return c
+
+    def to_dict(self) -> dict:
+        emb = {"scale": self.embedding_scale}
+        if self.bigram is not None:
+            emb["bigram"] = {"buckets": self.bigram.buckets, "mul_prev": self.bigram.mul_prev, "mul_cur": self.bigram.mul_cur}
+        layers = []
+        for l in self.layers:
+            m = l.mixer
+            if l.type == "latent_attention":
+                mixer = {"heads": m.heads, "dim": m.dim, "vdim": m.vdim, "kv_rank": m.kv_rank, "scale": m.scale}
+            else:
+                mixer = m.to_dict()
+            layers.append({"type": l.type, "mixer": mixer, "mlp": l.mlp.to_dict() if l.mlp else None})
+        d = {"architecture": "Fukatar", "vocab": self.vocab, "width": self.width, "embedding": emb, "norm": {"eps": self.norm_eps}, "layers": layers}
+        if self.logit_softcap:
+            d["logit_softcap"] = self.logit_softcap
+        return d

@@ -1,6 +1,8 @@
 // Kernels of libi64hip_dense.so for gated linear recurrences and mixtures of experts (include/i64h_dense.h):
 //   gla_gates_kernel   : query activation and bounded forget gate, in place on the projection rows
 //   gla_scan_kernel    : linear attention with a decay per key channel, a head's matrix in registers (16 lanes per value column)
+//   gdn_gates_kernel / gdn_scan_kernel : gated delta rule - unit-vector queries and keys, write strength and decay; the recurrence with the
+//                        correction S^T k summed over the DPP row before the write, the read-out after it
 //   route_topk_kernel  : softmax scores, corrected choice, groups of neighbours, top-k and normalised weights, one wave per row
 //   moe_plan_kernel    : (token, choice) pairs grouped by expert: offsets, the token of every grouped row, the row of every pair
 //   moe_combine_kernel : weighted sum of the chosen experts' rows, pass-through entries and the shared expert's row
@@ -106,6 +108,155 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(const i64h_gla_args p, co
             for (int k = 0; k < KPT; ++k) {
                 const float kk = HASK ? u.k[k] : 1.0f - u.f[k];
                 S[j][k] = fmaf(u.f[k], S[j][k], kk * u.v[j]);
+                part = fmaf(S[j][k], u.q[k], part);
+            }
+            part = group_sum(part, 16);
+            if (nlane == 0 && cbase + j < P) p.out[t * p.ldo + a * P + cbase + j] = part;
+        }
+    };
+    Tok A[GL_TG], B[GL_TG];
+#pragma unroll
+    for (int i = 0; i < GL_TG; ++i) fetch(r0 + i, A[i]);
+    for (int64_t t = r0; t < r1; t += 2 * GL_TG) {
+#pragma unroll
+        for (int i = 0; i < GL_TG; ++i) fetch(t + GL_TG + i, B[i]);
+#pragma unroll
+        for (int i = 0; i < GL_TG; ++i) step(t + i, A[i]);
+#pragma unroll
+        for (int i = 0; i < GL_TG; ++i) fetch(t + 2 * GL_TG + i, A[i]);
+#pragma unroll
+        for (int i = 0; i < GL_TG; ++i) step(t + GL_TG + i, B[i]);
+    }
+#pragma unroll
+    for (int j = 0; j < CPT; ++j) {
+        if (cbase + j >= P) continue;
+        float* dst = gS + (int64_t)(cbase + j) * N;
+        if (vec) {
+#pragma unroll
+            for (int k = 0; k < KPT; k += 4)
+                if (n0 + k < N) *(float4*)(dst + k) = make_float4(S[j][k], S[j][k + 1], S[j][k + 2], S[j][k + 3]);
+        } else {
+#pragma unroll
+            for (int k = 0; k < KPT; ++k)
+                if (n0 + k < N) dst[k] = S[j][k];
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------------------
+// Gated delta rule.  gdn_gates_kernel: one workgroup per token - a wave per query / key head makes the head a unit vector in place (the
+// query also scaled), and the first threads turn the raw gate projections into the write strength and the decay of every head.
+__device__ __forceinline__ float bl_softplus(float x) { return x > 20.0f ? x : log1pf(expf(x)); }
+
+__global__ __launch_bounds__(256) void gdn_gates_kernel(const i64h_gdn_args p) {
+    const int64_t t = blockIdx.x;
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+    float* row = p.X + t * p.ldx;
+    if (p.unit_eps >= 0.0f || p.q_scale != 1.0f) {
+        for (int u = wid; u < 2 * p.kv_heads; u += 4) {
+            const bool isq = u < p.kv_heads;
+            float* x = row + (isq ? p.q_off + u * p.dim : p.k_off + (u - p.kv_heads) * p.dim);
+            float s = 0.0f;
+            for (int d = lane; d < p.dim; d += 64) s += x[d] * x[d];
+            s = wave_sum(s);
+            float f = p.unit_eps >= 0.0f ? 1.0f / sqrtf(s + p.unit_eps) : 1.0f;
+            if (isq) f *= p.q_scale;
+            for (int d = lane; d < p.dim; d += 64) x[d] *= f;
+        }
+    }
+    for (int a = threadIdx.x; a < p.heads; a += 256) {
+        const float* r = p.R + t * p.ldr;
+        p.G[t * 2 * p.heads + a] = bl_sigmoid(r[p.b_off + a]);
+        p.G[t * 2 * p.heads + p.heads + a] = expf(-expf(p.A_log[a]) * bl_softplus(r[p.a_off + a] + p.dt_bias[a]));
+    }
+}
+
+// gdn_scan_kernel: the layout of gla_scan_kernel (one workgroup per (head, 16 * CPT value columns, run of rows); the 16 lanes of a DPP
+// row share CPT value columns and hold KPT key channels of each in registers).  Per token the state decays, the row sums S^T k with DPP
+// moves (every lane of the row ends with the sum), the correction along k is written, and a second row sum reads the state out with
+// the query - after the write.  No LDS and no barrier, the tokens of a run strictly in their order; loads run GL_TG tokens ahead.
+template <int KPT, int CPT>
+__global__ __launch_bounds__(256) void gdn_scan_kernel(const i64h_gdn_args p, const int ctiles, const int vec) {
+    const int N = p.dim, P = p.vdim;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int nlane = lane & 15, cl = lane >> 4;
+    const int a = blockIdx.x / ctiles, seg = blockIdx.y;
+    const int kh = a / (p.heads / p.kv_heads);
+    const int cbase = (blockIdx.x % ctiles) * 16 * CPT + (w * 4 + cl) * CPT;
+    const int64_t r0 = p.seg_start[seg], r1 = p.seg_start[seg + 1];
+    if (r1 <= r0) return;
+    const int n0 = nlane * KPT;
+    float S[CPT][KPT];
+    float* gS = p.state + ((int64_t)p.slot_ids[r0] * p.heads + a) * P * N + n0;      // + column * N
+    const bool fresh = p.positions[r0] == 0;
+#pragma unroll
+    for (int j = 0; j < CPT; ++j) {
+        const bool cok = cbase + j < P;
+        const float* src = gS + (int64_t)(cok ? cbase + j : 0) * N;
+#pragma unroll
+        for (int k = 0; k < KPT; ++k) S[j][k] = 0.0f;
+        if (!fresh && cok) {
+            if (vec) {
+#pragma unroll
+                for (int k = 0; k < KPT; k += 4)
+                    if (n0 + k < N) {
+                        const float4 v = *(const float4*)(src + k);
+                        S[j][k] = v.x, S[j][k + 1] = v.y, S[j][k + 2] = v.z, S[j][k + 3] = v.w;
+                    }
+            } else {
+#pragma unroll
+                for (int k = 0; k < KPT; ++k)
+                    if (n0 + k < N) S[j][k] = src[k];
+            }
+        }
+    }
+    const int qoff = p.q_off + kh * N + n0, koff = p.k_off + kh * N + n0;
+    struct Tok {
+        float q[KPT], k[KPT], v[CPT], beta, g;
+    };
+    auto fetch = [&](int64_t t, Tok& u) {
+        if (t >= r1) return;
+        const float* row = p.X + t * p.ldx;
+        if (vec) {      // KPT % 4 == 0 and every slice starts at a multiple of four floats and lies inside the row
+#pragma unroll
+            for (int k = 0; k < KPT; k += 4) {
+                float4 q = make_float4(0, 0, 0, 0), kk = q;
+                if (n0 + k < N) {
+                    q = *(const float4*)(row + qoff + k);
+                    kk = *(const float4*)(row + koff + k);
+                }
+                u.q[k] = q.x, u.q[k + 1] = q.y, u.q[k + 2] = q.z, u.q[k + 3] = q.w;
+                u.k[k] = kk.x, u.k[k + 1] = kk.y, u.k[k + 2] = kk.z, u.k[k + 3] = kk.w;
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < KPT; ++k) {
+                const bool ok = n0 + k < N;
+                u.q[k] = ok ? row[qoff + k] : 0.0f;
+                u.k[k] = ok ? row[koff + k] : 0.0f;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < CPT; ++j) u.v[j] = cbase + j < P ? row[p.v_off + a * P + cbase + j] : 0.0f;
+        u.beta = p.G[t * 2 * p.heads + a];
+        u.g = p.G[t * 2 * p.heads + p.heads + a];
+    };
+    auto step = [&](int64_t t, const Tok& u) {
+        if (t >= r1) return;
+#pragma unroll
+        for (int j = 0; j < CPT; ++j) {
+            float seen = 0.0f;
+#pragma unroll
+            for (int k = 0; k < KPT; ++k) {
+                S[j][k] *= u.g;
+                seen = fmaf(S[j][k], u.k[k], seen);
+            }
+            seen = group_sum(seen, 16);
+            const float d = u.beta * (u.v[j] - seen);
+            float part = 0.0f;
+#pragma unroll
+            for (int k = 0; k < KPT; ++k) {
+                S[j][k] = fmaf(u.k[k], d, S[j][k]);
                 part = fmaf(S[j][k], u.q[k], part);
             }
             part = group_sum(part, 16);
@@ -362,6 +513,53 @@ int i64h_gla_scan(const i64h_gla_args* dp, void* stream) {
         if (hask) { GLA_PICK(1, true) } else { GLA_PICK(1, false) }
     }
 #undef GLA_PICK
+    I64H_CHECK_LAUNCH();
+    return 0;
+}
+
+static int gdn_check(const i64h_gdn_args& d, const char* what) {
+    I64H_CHECK_ARG(d.heads > 0 && d.kv_heads > 0 && d.heads % d.kv_heads == 0 && d.dim > 0 && d.vdim > 0 && d.n >= 0, "%s: heads %d, query / key heads %d, dim %d, vdim %d",
+                   what, d.heads, d.kv_heads, d.dim, d.vdim);
+    I64H_CHECK_ARG(d.X && d.G && d.q_off >= 0 && d.k_off >= 0 && d.v_off >= 0, "%s: null operand or negative column", what);
+    return 0;
+}
+
+int i64h_gdn_gates(const i64h_gdn_args* dp, void* stream) {
+    I64H_CHECK_ARG(dp != nullptr, "gdn_gates: no descriptor");
+    const i64h_gdn_args& d = *dp;
+    if (gdn_check(d, "gdn_gates")) return 1;
+    I64H_CHECK_ARG(d.R && d.A_log && d.dt_bias && d.b_off >= 0 && d.a_off >= 0, "gdn_gates: null operand or negative column");
+    if (d.n == 0) return 0;
+    hipLaunchKernelGGL(gdn_gates_kernel, dim3((unsigned)d.n), dim3(256), 0, (hipStream_t)stream, d);
+    I64H_CHECK_LAUNCH();
+    return 0;
+}
+
+int i64h_gdn_scan(const i64h_gdn_args* dp, void* stream) {
+    I64H_CHECK_ARG(dp != nullptr, "gdn_scan: no descriptor");
+    const i64h_gdn_args& d = *dp;
+    if (gdn_check(d, "gdn_scan")) return 1;
+    I64H_CHECK_ARG(d.seg_start && d.positions && d.slot_ids && d.state && d.out, "gdn_scan: null operand");
+    I64H_CHECK_ARG(d.dim <= 16 * 16, "gdn_scan: dim %d above 256", d.dim);
+    I64H_CHECK_ARG(d.nseg <= 65535, "gdn_scan: %d runs in one launch", d.nseg);
+    if (d.nseg <= 0 || d.n == 0) return 0;
+    const int kpt = (d.dim + 15) / 16;
+    // columns per lane: query and key are loaded once for both - unless the launch would then leave most of the chip idle
+    const int cpt = (d.vdim > 16 && (int64_t)d.heads * ((d.vdim + 31) / 32) * d.nseg >= 512) ? 2 : 1;
+    const int ctiles = (d.vdim + 16 * cpt - 1) / (16 * cpt);
+    const dim3 grid((unsigned)(d.heads * ctiles), (unsigned)d.nseg);
+    auto launch = [&](auto kern, int K) {
+        const int vec = K % 4 == 0 && d.dim % 4 == 0 && d.ldx % 4 == 0 && d.q_off % 4 == 0 && d.k_off % 4 == 0 && (uintptr_t)d.X % 16 == 0 && (uintptr_t)d.state % 16 == 0;
+        hipLaunchKernelGGL(kern, grid, dim3(256), 0, (hipStream_t)stream, d, ctiles, vec);
+    };
+#define GDN_PICK(C)                                          \
+    if (kpt <= 1) launch(gdn_scan_kernel<1, C>, 1);          \
+    else if (kpt <= 2) launch(gdn_scan_kernel<2, C>, 2);     \
+    else if (kpt <= 4) launch(gdn_scan_kernel<4, C>, 4);     \
+    else if (kpt <= 8) launch(gdn_scan_kernel<8, C>, 8);     \
+    else launch(gdn_scan_kernel<16, C>, 16);
+    if (cpt == 2) { GDN_PICK(2) } else { GDN_PICK(1) }
+#undef GDN_PICK
     I64H_CHECK_LAUNCH();
     return 0;
 }

@@ -42,6 +42,7 @@ __device__ __forceinline__ float dn_epilogue(const i64h_linear& p, float acc, fl
     if (EPI == I64H_EPI_SILU_MUL) return acc * dn_sigmoid(acc) * acc2;
     if (p.bias) acc += p.bias[b * p.bias_batch + c];
     if (EPI == I64H_EPI_XIELU) return dn_xielu(acc, p.act_a, p.act_b);
+    if (EPI == I64H_EPI_RELU_SQ) return acc > 0.0f ? acc * acc : 0.0f;
     if (EPI == I64H_EPI_GELU_ERF) return dn_gelu_erf(acc);
     if (EPI == I64H_EPI_SCALE) return acc * p.scale;
     if (EPI == I64H_EPI_MUL_SIGMOID) return acc * dn_sigmoid(p.E[b * p.e_batch + r * p.lde + c]);
@@ -689,6 +690,7 @@ static void launch_tile(const i64h_linear& d, dim3 grid, hipStream_t s, int vecA
         case I64H_EPI_SOFTCAP: hipLaunchKernelGGL((linear_tile_kernel<EXACT, I64H_EPI_SOFTCAP>), grid, dim3(256), 0, s, d, vecA, vecW); break;
         case I64H_EPI_GELU_ERF: hipLaunchKernelGGL((linear_tile_kernel<EXACT, I64H_EPI_GELU_ERF>), grid, dim3(256), 0, s, d, vecA, vecW); break;
         case I64H_EPI_XIELU: hipLaunchKernelGGL((linear_tile_kernel<EXACT, I64H_EPI_XIELU>), grid, dim3(256), 0, s, d, vecA, vecW); break;
+        case I64H_EPI_RELU_SQ: hipLaunchKernelGGL((linear_tile_kernel<EXACT, I64H_EPI_RELU_SQ>), grid, dim3(256), 0, s, d, vecA, vecW); break;
         case I64H_EPI_SCALE: hipLaunchKernelGGL((linear_tile_kernel<EXACT, I64H_EPI_SCALE>), grid, dim3(256), 0, s, d, vecA, vecW); break;
         default: hipLaunchKernelGGL((linear_tile_kernel<EXACT, I64H_EPI_STORE>), grid, dim3(256), 0, s, d, vecA, vecW); break;
     }
@@ -715,7 +717,7 @@ int i64h_linear_run(const i64h_linear* dp, void* stream) {
     const i64h_linear& d = *dp;
     I64H_CHECK_ARG(d.M >= 0 && d.N > 0 && d.K > 0 && d.batch > 0, "linear: bad sizes M=%lld N=%d K=%d batch=%d", (long long)d.M, d.N, d.K, d.batch);
     I64H_CHECK_ARG(d.A && d.W && d.C, "linear: null operand");
-    I64H_CHECK_ARG(d.epilogue >= 0 && d.epilogue <= 7, "linear: epilogue %d", d.epilogue);
+    I64H_CHECK_ARG(d.epilogue >= 0 && d.epilogue <= I64H_EPI_RELU_SQ, "linear: epilogue %d", d.epilogue);
     I64H_CHECK_ARG(d.epilogue != I64H_EPI_MUL_SIGMOID || d.E, "linear: the sigmoid epilogue needs E");
     I64H_CHECK_ARG(d.epilogue != I64H_EPI_SOFTCAP || d.softcap > 0.0f, "linear: soft cap %g", (double)d.softcap);
     I64H_CHECK_ARG(!dn_dual(d.epilogue) || !d.bias, "linear: the gate / up epilogues take no bias");
@@ -737,6 +739,7 @@ int i64h_linear_run(const i64h_linear* dp, void* stream) {
             case I64H_EPI_SOFTCAP: hipLaunchKernelGGL((linear_skinny_kernel<I64H_EPI_SOFTCAP>), grid, dim3(256), lds, s, d, cpb); break;
             case I64H_EPI_GELU_ERF: hipLaunchKernelGGL((linear_skinny_kernel<I64H_EPI_GELU_ERF>), grid, dim3(256), lds, s, d, cpb); break;
             case I64H_EPI_XIELU: hipLaunchKernelGGL((linear_skinny_kernel<I64H_EPI_XIELU>), grid, dim3(256), lds, s, d, cpb); break;
+            case I64H_EPI_RELU_SQ: hipLaunchKernelGGL((linear_skinny_kernel<I64H_EPI_RELU_SQ>), grid, dim3(256), lds, s, d, cpb); break;
             case I64H_EPI_SCALE: hipLaunchKernelGGL((linear_skinny_kernel<I64H_EPI_SCALE>), grid, dim3(256), lds, s, d, cpb); break;
             default: hipLaunchKernelGGL((linear_skinny_kernel<I64H_EPI_STORE>), grid, dim3(256), lds, s, d, cpb); break;
         }
@@ -753,6 +756,7 @@ int i64h_linear_run(const i64h_linear* dp, void* stream) {
             case I64H_EPI_SOFTCAP: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_SOFTCAP, 8>), grid, dim3(512), 0, s, d); break;
             case I64H_EPI_GELU_ERF: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_GELU_ERF, 8>), grid, dim3(512), 0, s, d); break;
             case I64H_EPI_XIELU: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_XIELU, 8>), grid, dim3(512), 0, s, d); break;
+            case I64H_EPI_RELU_SQ: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_RELU_SQ, 8>), grid, dim3(512), 0, s, d); break;
             case I64H_EPI_SCALE: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_SCALE, 8>), grid, dim3(512), 0, s, d); break;
             default: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_STORE, 8>), grid, dim3(512), 0, s, d); break;
         }
@@ -769,6 +773,7 @@ int i64h_linear_run(const i64h_linear* dp, void* stream) {
             case I64H_EPI_SOFTCAP: hipLaunchKernelGGL((linear_tile128_kernel<I64H_EPI_SOFTCAP>), grid, dim3(256), 0, s, d, vecA, vecW); break;
             case I64H_EPI_GELU_ERF: hipLaunchKernelGGL((linear_tile128_kernel<I64H_EPI_GELU_ERF>), grid, dim3(256), 0, s, d, vecA, vecW); break;
             case I64H_EPI_XIELU: hipLaunchKernelGGL((linear_tile128_kernel<I64H_EPI_XIELU>), grid, dim3(256), 0, s, d, vecA, vecW); break;
+            case I64H_EPI_RELU_SQ: hipLaunchKernelGGL((linear_tile128_kernel<I64H_EPI_RELU_SQ>), grid, dim3(256), 0, s, d, vecA, vecW); break;
             case I64H_EPI_SCALE: hipLaunchKernelGGL((linear_tile128_kernel<I64H_EPI_SCALE>), grid, dim3(256), 0, s, d, vecA, vecW); break;
             default: hipLaunchKernelGGL((linear_tile128_kernel<I64H_EPI_STORE>), grid, dim3(256), 0, s, d, vecA, vecW); break;
         }

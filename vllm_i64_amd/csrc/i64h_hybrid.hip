@@ -52,7 +52,7 @@ __global__ __launch_bounds__(256) void embed_bigram_kernel(const i64h_embed_bigr
     const int64_t plane = p.n * (int64_t)W;
     const int64_t prow = p.pos_table ? min(max((int64_t)p.positions[t], (int64_t)0), p.pos_rows - 1) : 0;
     for (int c = threadIdx.x; c < W; c += 256) {
-        float v = hy_bf16(p.table, id * W + c);
+        float v = hy_bf16(p.table, id * W + c) * p.scale;
         if (p.pos_table) v += hy_bf16(p.pos_table, prow * W + c);
         if (brow >= 0) v += hy_bf16(p.bigram, brow * W + c);
         for (int s = 0; s < p.copies; ++s) p.out[s * plane + t * W + c] = v;
@@ -99,15 +99,37 @@ __global__ __launch_bounds__(256) void streams_kernel(const i64h_streams_args p)
         a = hy_block_sum(a, red);
         ya = sqrtf(a / (float)W + p.y_eps);     // divided by, as the norm in front is
     }
-    float ss = 0.0f;
+    // the result as the residual receives it: both side-by-side parts normed and averaged, or the one result with its own norm, or as it is
+    auto result = [&](int c) -> float {
+        float v = p.y[m * p.ldy + c];
+        if (p.y2) v = 0.5f * (v * ya * p.yn_w[c] + p.y2[m * p.ldy2 + c] * yb * p.y2n_w[c]);
+        else if (p.yn_w) v = v / ya * p.yn_w[c];
+        return v;
+    };
+    float pmean = 0.0f, pden = 1.0f;
+    if (p.y && p.post_w) {   // a norm over the whole result: the row waits in LDS, mean first, then the squared deviations
+        float a = 0.0f;
+        for (int c = tid; c < W; c += 256) {
+            const float v = result(c);
+            sv[c] = v;
+            a += v;
+        }
+        if (p.post_center) pmean = hy_block_sum(a, red) / (float)W;
+        float b = 0.0f;
+        for (int c = tid; c < W; c += 256) {
+            const float u = sv[c] - pmean;
+            b += u * u;
+        }
+        b = hy_block_sum(b, red);
+        pden = sqrtf(b / (float)W + p.y_eps);
+    }
+    float ss = 0.0f, su = 0.0f;
     for (int c = tid; c < W; c += 256) {
         float x[HY_MAX_STREAMS];
 #pragma unroll
         for (int s = 0; s < HY_MAX_STREAMS; ++s) x[s] = s < S ? xs[s * plane + c] : 0.0f;
         if (p.y) {
-            float v = p.y[m * p.ldy + c];
-            if (p.y2) v = 0.5f * (v * ya * p.yn_w[c] + p.y2[m * p.ldy2 + c] * yb * p.y2n_w[c]);
-            else if (p.yn_w) v = v / ya * p.yn_w[c];
+            const float v = p.post_w ? (sv[c] - pmean) / pden * p.post_w[c] : result(c);
             float nx[HY_MAX_STREAMS];
 #pragma unroll
             for (int t = 0; t < HY_MAX_STREAMS; ++t) {
@@ -133,12 +155,22 @@ __global__ __launch_bounds__(256) void streams_kernel(const i64h_streams_args p)
                 if (s < S) u += (p.in_w ? p.in_w[s] : 1.0f) * x[s];
             sv[c] = u;
             ss += u * u;
+            su += u;
         }
     }
     if (!p.h) return;
+    float mean = 0.0f;
+    if (p.h_center) {        // the centred norm: the squared deviations from the mean, summed in a pass of their own
+        mean = hy_block_sum(su, red) / (float)W;
+        ss = 0.0f;
+        for (int c = tid; c < W; c += 256) {
+            const float u = sv[c] - mean;
+            ss += u * u;
+        }
+    }
     ss = hy_block_sum(ss, red);
     const float den = sqrtf(ss / (float)W + p.eps);
-    for (int c = tid; c < W; c += 256) p.h[m * W + c] = sv[c] / den * p.norm_w[p.norm_w_len == 1 ? 0 : c];
+    for (int c = tid; c < W; c += 256) p.h[m * W + c] = (sv[c] - mean) / den * p.norm_w[p.norm_w_len == 1 ? 0 : c];
 }
 
 // ---------------------------------------------------------------------------------------------------------------------------
@@ -343,7 +375,7 @@ __global__ __launch_bounds__(256) void gate_norm_kernel(const i64h_gate_norm_arg
     const int W = p.width;
     for (int c = tid; c < W; c += 256) {
         float v = p.y[m * p.ldy + c];
-        if (p.z) v *= hy_silu(p.z[m * p.ldz + c]);
+        if (p.z && !p.gate_after) v *= hy_silu(p.z[m * p.ldz + c]);
         sv[c] = v;
     }
     __syncthreads();
@@ -358,7 +390,11 @@ __global__ __launch_bounds__(256) void gate_norm_kernel(const i64h_gate_norm_arg
         if (lane == 0) sv[W + g] = sqrtf(s / (float)gs + p.eps);
     }
     __syncthreads();
-    for (int c = tid; c < W; c += 256) p.out[m * p.ldo + c] = sv[c] / sv[W + c / gs] * p.w[c];
+    for (int c = tid; c < W; c += 256) {
+        float v = sv[c] / sv[W + c / gs] * p.w[p.w_len > 0 ? c % p.w_len : c];
+        if (p.z && p.gate_after) v *= hy_silu(p.z[m * p.ldz + c]);
+        p.out[m * p.ldo + c] = v;
+    }
 }
 
 // ---------------------------------------------------------------------------------------------------------------------------
@@ -488,6 +524,7 @@ __global__ __launch_bounds__(256) void kattn_row_kernel(const i64h_kattn_args p)
             float dot = 0.0f;
             for (int d = 0; d < dim; ++d) dot += sq[wid][d] * (float)kr[d];
             s = p.kscale ? dot * p.kscale[row] : dot;
+            if (p.softcap > 0.0f) s = p.softcap * tanhf(s / p.softcap);
             if (p.bias) s += p.bias[(int64_t)min(pos - j, p.bias_rows - 1) * p.heads + h];
         }
         srow[wid][lane] = row;
@@ -534,6 +571,135 @@ __global__ __launch_bounds__(256) void kv_prep_kernel(const i64h_kv_prep_args p)
         const float v = d < p.vdim ? row[p.v_off + g * p.vdim + d] : row[p.k_off + g * p.dim + d - p.vdim];
         if (p.cache_dtype == 0) ((float*)p.cache)[cr * nk + c] = v;
         else ((__bf16*)p.cache)[cr * nk + c] = (__bf16)v;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------------------
+// [q | k | v] projections -> whole-row norms, rotation (two pair layouts, a part of every head), per-head norms, rotated values ->
+// the paged cache row [v | k] per key head and the query rows [0 | q * scale].  One workgroup per token; the normed and rotated
+// queries and keys wait in LDS for the per-head sums.
+__device__ __forceinline__ void rot_pair(int d, int dims, int interleaved, int& a, int& b, int& i, bool& second) {
+    // the pair of dimension d < dims: a the first member, b the second, i the pair's index; second: d is b
+    if (interleaved) {
+        i = d >> 1, a = d & ~1, b = d | 1, second = d & 1;
+    } else {
+        const int half = dims >> 1;
+        second = d >= half, i = second ? d - half : d, a = i, b = i + half;
+    }
+}
+
+__global__ __launch_bounds__(256) void rot_prep_kernel(const i64h_rot_prep_args p) {
+    extern __shared__ float sv[];   // [heads * dim] queries, [kv_heads * dim] keys, [heads + kv_heads] 1 / rms per head, 4 for reductions
+    const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
+    const int64_t t = blockIdx.x;
+    const int dim = p.dim, vd = p.vdim, gs = vd + dim;
+    const int nq = p.heads * dim, nk = p.kv_heads * dim;
+    float* inv = sv + nq + nk;
+    float* red = inv + p.heads + p.kv_heads;
+    const float* q = p.P + t * p.ldp + p.q_off;
+    const float* k = p.P + t * p.ldp + p.k_off;
+    const float* v = p.P + t * p.ldp + p.v_off;
+    const int pos = p.positions[t];
+    const float fpos = (float)pos;
+    float qr = 1.0f, kr = 1.0f;
+    if (p.q_norm_w) {
+        float a = 0.0f, b = 0.0f;
+        for (int c = tid; c < nq; c += 256) a += q[c] * q[c];
+        for (int c = tid; c < nk; c += 256) b += k[c] * k[c];
+        a = hy_block_sum(a, red);
+        b = hy_block_sum(b, red);
+        qr = 1.0f / sqrtf(a / (float)nq + p.eps);
+        kr = 1.0f / sqrtf(b / (float)nk + p.eps);
+    }
+    for (int c = tid; c < nq + nk; c += 256) {
+        const bool isq = c < nq;
+        const int e = isq ? c : c - nq;
+        const int h0 = (e / dim) * dim, d = e % dim;
+        const float* src = isq ? q : k;
+        const float* nw = isq ? p.q_norm_w : p.k_norm_w;
+        const float r = isq ? qr : kr;
+        auto val = [&](int idx) { return nw ? src[idx] * r * nw[idx] : src[idx]; };
+        float o;
+        if (d < p.rot_dims) {
+            int a, b, i;
+            bool second;
+            rot_pair(d, p.rot_dims, p.interleaved, a, b, i, second);
+            float sn, cs;
+            sincosf(fpos * p.inv_freq[i], &sn, &cs);
+            sn *= p.rot_mult, cs *= p.rot_mult;
+            const float u = val(h0 + a), w = val(h0 + b);
+            o = second ? w * cs + u * sn : u * cs - w * sn;
+        } else {
+            o = val(h0 + d);
+        }
+        sv[c] = o;
+    }
+    __syncthreads();
+    if (p.head_norm) {
+        for (int h = wid; h < p.heads + p.kv_heads; h += 4) {
+            float s = 0.0f;
+            for (int d = lane; d < dim; d += 64) s += sv[h * dim + d] * sv[h * dim + d];
+            s = wave_sum(s);
+            if (lane == 0) inv[h] = 1.0f / sqrtf(s / (float)dim + p.eps);
+        }
+        __syncthreads();
+    }
+    float* Q = p.Q + t * p.heads * gs;
+    for (int c = tid; c < p.heads * gs; c += 256) {
+        const int h = c / gs, d = c % gs;
+        float o = 0.0f;
+        if (d >= vd) {
+            o = sv[h * dim + d - vd];
+            if (p.head_norm) o *= inv[h];
+            o *= p.scale;
+        }
+        Q[c] = o;
+    }
+    const int64_t cr = cache_row(p.block_table, p.max_blocks_per_seq, p.block_size, p.slot_ids[t], pos);
+    const int nkv = p.kv_heads * gs;
+    for (int c = tid; c < nkv; c += 256) {
+        const int g = c / gs, d = c % gs;
+        float o;
+        if (d >= vd) {
+            o = sv[nq + g * dim + d - vd];
+            if (p.head_norm) o *= inv[p.heads + g];
+        } else if (p.v_freq) {
+            int a, b, i;
+            bool second;
+            rot_pair(d, vd, p.interleaved, a, b, i, second);
+            float sn, cs;
+            sincosf(fpos * p.v_freq[i], &sn, &cs);
+            const float u = v[g * vd + a], w = v[g * vd + b];
+            o = second ? w * cs + u * sn : u * cs - w * sn;
+        } else {
+            o = v[g * vd + d];
+        }
+        if (p.cache_dtype == 0) ((float*)p.cache)[cr * nkv + c] = o;
+        else ((__bf16*)p.cache)[cr * nkv + c] = (__bf16)o;
+    }
+}
+
+// the attention output of every head turned back by the row's own position and multiplied by the head's sigmoid gate, in place:
+// a thread takes whole pairs
+__global__ __launch_bounds__(256) void rot_post_kernel(const i64h_rot_post_args p) {
+    const int64_t t = blockIdx.x;
+    const int vd = p.vdim, half = vd >> 1;
+    const float fpos = (float)p.positions[t];
+    float* O = p.O + t * p.heads * vd;
+    const int items = p.v_freq ? p.heads * half : p.heads * vd;
+    for (int e = threadIdx.x; e < items; e += 256) {
+        if (p.v_freq) {
+            const int h = e / half, i = e % half;
+            const int a = p.interleaved ? 2 * i : i, b = p.interleaved ? 2 * i + 1 : i + half;
+            const float g = p.gate ? hy_sigmoid(p.gate[t * p.ldg + h]) : 1.0f;
+            float sn, cs;
+            sincosf(fpos * p.v_freq[i], &sn, &cs);
+            const float u = O[h * vd + a], w = O[h * vd + b];
+            O[h * vd + a] = (u * cs + w * sn) * g;      // the turn by the negative angle
+            O[h * vd + b] = (w * cs - u * sn) * g;
+        } else {
+            O[e] *= hy_sigmoid(p.gate[t * p.ldg + e / vd]);
+        }
     }
 }
 
@@ -701,7 +867,7 @@ int i64h_kattn(const i64h_kattn_args* dp, void* stream) {
         a.block_size = d.block_size, a.slot_ids = d.slot_ids, a.positions = d.positions, a.window = 0, a.scale = 1.0f, a.out = d.out, a.n = d.n;
         a.heads = d.heads, a.kv_rank = vals, a.rot_dim = gs - vals, a.mode = d.mode == 3 ? 3 : 2, a.splits = d.splits, a.workspace = d.workspace;
         a.row_stride = d.kv_heads * gs, a.kv_groups = d.kv_heads, a.chunk = d.chunk, a.kscale = d.kscale, a.bias = d.bias, a.bias_rows = d.bias_rows;
-        a.sink = d.sink;
+        a.sink = d.sink, a.softcap = d.softcap;
         a.key_off = d.vdim > 0 ? d.vdim : 0;
         return i64h_latent_attn(&a, stream);
     }
@@ -722,6 +888,35 @@ int i64h_kv_prep(const i64h_kv_prep_args* dp, void* stream) {
     I64H_CHECK_ARG(!d.cache || (d.block_table && d.block_size > 0 && d.max_blocks_per_seq > 0 && (d.cache_dtype == 0 || d.cache_dtype == 2)), "kv_prep: bad paging or cache type");
     if (d.n == 0) return 0;
     hipLaunchKernelGGL(kv_prep_kernel, dim3((unsigned)d.n), dim3(256), 0, (hipStream_t)stream, d);
+    I64H_CHECK_LAUNCH();
+    return 0;
+}
+
+int i64h_rot_prep(const i64h_rot_prep_args* dp, void* stream) {
+    I64H_CHECK_ARG(dp != nullptr, "rot_prep: no descriptor");
+    const i64h_rot_prep_args& d = *dp;
+    I64H_CHECK_ARG(d.heads > 0 && d.kv_heads > 0 && d.heads % d.kv_heads == 0 && d.dim > 0 && d.vdim > 0, "rot_prep: heads %d, kv heads %d, dim %d, vdim %d",
+                   d.heads, d.kv_heads, d.dim, d.vdim);
+    I64H_CHECK_ARG(d.rot_dims >= 0 && d.rot_dims <= d.dim && d.rot_dims % 2 == 0 && (d.rot_dims == 0 || d.inv_freq), "rot_prep: %d rotated dimensions of %d", d.rot_dims, d.dim);
+    I64H_CHECK_ARG(!d.v_freq || d.vdim % 2 == 0, "rot_prep: rotated values of an odd size %d", d.vdim);
+    I64H_CHECK_ARG((d.q_norm_w == nullptr) == (d.k_norm_w == nullptr), "rot_prep: the whole-row norms come together");
+    I64H_CHECK_ARG(d.P && d.Q && d.positions && d.slot_ids && d.block_table && d.cache, "rot_prep: null operand");
+    I64H_CHECK_ARG(d.block_size > 0 && d.max_blocks_per_seq > 0 && (d.cache_dtype == 0 || d.cache_dtype == 2), "rot_prep: bad paging or cache type");
+    const size_t lds = ((size_t)(d.heads + d.kv_heads) * (d.dim + 1) + 4) * 4;
+    I64H_CHECK_ARG(lds <= 64 * 1024, "rot_prep: %d + %d heads of %d values do not fit the kernel's LDS buffer", d.heads, d.kv_heads, d.dim);
+    if (d.n == 0) return 0;
+    hipLaunchKernelGGL(rot_prep_kernel, dim3((unsigned)d.n), dim3(256), lds, (hipStream_t)stream, d);
+    I64H_CHECK_LAUNCH();
+    return 0;
+}
+
+int i64h_rot_post(const i64h_rot_post_args* dp, void* stream) {
+    I64H_CHECK_ARG(dp != nullptr, "rot_post: no descriptor");
+    const i64h_rot_post_args& d = *dp;
+    I64H_CHECK_ARG(d.heads > 0 && d.vdim > 0 && (!d.v_freq || d.vdim % 2 == 0), "rot_post: heads %d, vdim %d", d.heads, d.vdim);
+    I64H_CHECK_ARG(d.O && d.positions && (d.v_freq || d.gate), "rot_post: null operand or nothing to do");
+    if (d.n == 0) return 0;
+    hipLaunchKernelGGL(rot_post_kernel, dim3((unsigned)d.n), dim3(256), 0, (hipStream_t)stream, d);
     I64H_CHECK_LAUNCH();
     return 0;
 }

@@ -79,7 +79,8 @@ __global__ __launch_bounds__(256) void latent_attn_row_kernel(const i64h_latent_
     __syncthreads();
     const int j0 = p.window > 0 ? max(0, pos - p.window + 1) : 0;
     const int32_t* bt = p.block_table + (int64_t)slot * p.max_blocks_per_seq;
-    float m = -INFINITY, l = 0.0f, acc[LT_MAXC];
+    // the sink: one more score (a learned one per head, or zero) that counts in the denominator and carries no value
+    float m = p.sink ? (p.sink_w ? p.sink_w[h] : 0.0f) : -INFINITY, l = p.sink ? 1.0f : 0.0f, acc[LT_MAXC];
 #pragma unroll
     for (int i = 0; i < LT_MAXC; ++i) acc[i] = 0.0f;
     for (int jb = j0; jb <= pos; jb += 64) {
@@ -114,6 +115,7 @@ __global__ __launch_bounds__(256) void latent_attn_row_kernel(const i64h_latent_
                 for (int d = 0; d < D; ++d) s += sq[d] * __uint_as_float((uint32_t)kr[d] << 16);
             }
         }
+        if (p.softcap > 0.0f) s = p.softcap * tanhf(s / p.softcap);
         s = valid ? s : -INFINITY;
         const float mn = fmaxf(m, wave_max(s));
         const float alpha = expf(m - mn);
@@ -237,13 +239,14 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, KD > 4 ? 
     int lor[4], hrow[4];   // per row of the tile: the first position it sees, its head (for the bias table)
     const bool sink = p.sink && split == 0;     // the extra score of zero counts once: in the first share of the keys
     __syncthreads();
+    const float capl = p.softcap * 1.4426950408889634f;     // the cap in the units of the scores (powers of two)
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-        mrow[g] = sink ? 0.0f : -INFINITY;
-        lrow[g] = sink ? 1.0f : 0.0f;
         const int pp = info[kg * 4 + g];
         lor[g] = p.chunk > 0 ? (max(pp, 0) / p.chunk) * p.chunk : (win > 0 ? max(0, pp - win + 1) : 0);
         hrow[g] = min(row_tiles ? hbase : hbase + kg * 4 + g, H - 1);
+        mrow[g] = sink ? (p.sink_w ? p.sink_w[hrow[g]] * 1.4426950408889634f : 0.0f) : -INFINITY;
+        lrow[g] = sink ? 1.0f : 0.0f;
     }
     const uint16_t* cache = (const uint16_t*)p.cache;
     int s0 = 0;
@@ -307,6 +310,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, KD > 4 ? 
                     const int j = kb + 16 * b + n;
                     const bool vis = in_run && j <= pr && j >= lor[g];
                     float sc = S[b][g] * ksc[b];
+                    if (capl > 0.0f) sc = capl * tanhf(sc / capl);
                     if (p.bias) sc += 1.4426950408889634f * p.bias[(int64_t)min(max(pr - j, 0), p.bias_rows - 1) * H + hrow[g]];
                     sv[b] = vis ? sc : -INFINITY;
                 }
@@ -453,11 +457,12 @@ __global__ __launch_bounds__(64) void latent_attn_mfma_decode_kernel(const i64h_
     float mrow[4], lrow[4];
     int hrow[4];
     const bool sink = p.sink && split == 0;     // the extra score of zero counts once: in the first share of the keys
+    const float capl = p.softcap * 1.4426950408889634f;     // the cap in the units of the scores (powers of two)
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-        mrow[g] = sink ? 0.0f : -INFINITY;
-        lrow[g] = sink ? 1.0f : 0.0f;
         hrow[g] = min(head0 + kg * 4 + g, H - 1);
+        mrow[g] = sink ? (p.sink_w ? p.sink_w[hrow[g]] * 1.4426950408889634f : 0.0f) : -INFINITY;
+        lrow[g] = sink ? 1.0f : 0.0f;
     }
     int it = 0;
     for (int kb = kb0; kb <= hi; kb += step, ++it) {
@@ -499,6 +504,7 @@ __global__ __launch_bounds__(64) void latent_attn_mfma_decode_kernel(const i64h_
             for (int b = 0; b < 2; ++b) {
                 const int j = kb + 16 * b + n;
                 float sc = S[b][g] * ksc[b];
+                if (capl > 0.0f) sc = capl * tanhf(sc / capl);
                 if (p.bias) sc += 1.4426950408889634f * p.bias[(int64_t)min(max(pos - j, 0), p.bias_rows - 1) * H + hrow[g]];
                 sv[b] = (j <= pos && j >= lo) ? sc : -INFINITY;
             }
@@ -632,8 +638,9 @@ int i64h_latent_attn(const i64h_latent_attn_args* dp, void* stream) {
     const int D = d.kv_rank + d.rot_dim;
     const bool mfma_ok = d.cache_dtype == 2 && D % 8 == 0 && d.kv_rank % 16 == 0 && d.kv_rank <= 16 * LT_NB && D <= 32 * LT_KD &&
                          (uintptr_t)d.Q % 16 == 0 && (uintptr_t)d.cache % 16 == 0 && d.row_stride % 8 == 0;
-    I64H_CHECK_ARG(mfma_ok || d.mode == 1 || (d.kv_groups <= 1 && d.row_stride <= 0 && d.chunk <= 0 && !d.kscale && !d.bias && !d.sink),
-                   "latent_attn: key heads, chunks, key scales, bias and sink are built for the matrix-core form only");
+    I64H_CHECK_ARG(mfma_ok || (d.kv_groups <= 1 && d.row_stride <= 0 && d.chunk <= 0 && !d.kscale && !d.bias),
+                   "latent_attn: key heads, chunks, key scales and bias are built for the matrix-core form only");
+    I64H_CHECK_ARG(!d.sink_w || d.sink, "latent_attn: sink scores without the sink");
     if (d.mode != 1 && mfma_ok) {
         const int row_tiles = d.mode == 3;
         const int G = d.kv_groups > 1 ? d.kv_groups : 1;

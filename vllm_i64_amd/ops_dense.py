@@ -11,7 +11,7 @@ from . import _lib
 from ._lib import call_dense, ptr
 from .ops import _chk, _stream
 
-EPI_STORE, EPI_GELU_MUL, EPI_MUL_SIGMOID, EPI_SOFTCAP, EPI_GELU_ERF, EPI_SCALE, EPI_SILU_MUL, EPI_XIELU = 0, 1, 2, 3, 4, 5, 6, 7
+EPI_STORE, EPI_GELU_MUL, EPI_MUL_SIGMOID, EPI_SOFTCAP, EPI_GELU_ERF, EPI_SCALE, EPI_SILU_MUL, EPI_XIELU, EPI_RELU_SQ = 0, 1, 2, 3, 4, 5, 6, 7, 8
 _DUAL = (EPI_GELU_MUL, EPI_SILU_MUL)
 CACHE_DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 2}
 
@@ -121,11 +121,17 @@ def latent_prep(p: torch.Tensor, *, q_off: int, dkv_off: int, heads: int, dim: i
 
 def latent_attn(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor, slot_ids: torch.Tensor, positions: torch.Tensor, *,
                 window: int, scale: float, heads: int, kv_rank: int, rot_dim: int, out: torch.Tensor, n: Optional[int] = None,
-                mode: int = 0, splits: int = 1, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+                mode: int = 0, splits: int = 1, workspace: Optional[torch.Tensor] = None, sink: Optional[torch.Tensor] = None,
+                softcap: float = 0.0) -> torch.Tensor:
+    """See i64h_latent_attn.  sink fp32 [heads]: a learned extra score per head in the softmax's denominator."""
     _chk(q, torch.float32, "q"), _chk(out, torch.float32, "out"), _chk(cache, None, "cache")
     _chk(positions, torch.int32, "positions"), _chk(slot_ids, torch.int32, "slot_ids"), _chk(block_table, torch.int32, "block_table")
     rows = int(n if n is not None else positions.numel())
     D = kv_rank + rot_dim
+    if sink is not None:
+        _chk(sink, torch.float32, "sink")
+        if sink.numel() != heads:
+            raise _lib.I64HError("latent_attn: the sink scores are not [heads]")
     if cache.shape[-1] != D or q.numel() < rows * heads * D or out.numel() < rows * heads * kv_rank:
         raise _lib.I64HError("latent_attn: cache / query / output shapes do not fit the sizes")
     if splits > 1:
@@ -138,7 +144,8 @@ def latent_attn(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor,
     d = _lib.LatentAttn(Q=ptr(q), cache=ptr(cache), cache_dtype=CACHE_DTYPE_CODE[cache.dtype], block_table=ptr(block_table),
                         max_blocks_per_seq=block_table.shape[1], block_size=cache.shape[-2], slot_ids=ptr(slot_ids), positions=ptr(positions),
                         window=int(window), scale=float(scale), out=ptr(out), n=rows, heads=heads, kv_rank=kv_rank, rot_dim=rot_dim, mode=mode,
-                        splits=int(splits) if splits > 1 else 1, workspace=ptr(workspace) if splits > 1 else 0)
+                        splits=int(splits) if splits > 1 else 1, workspace=ptr(workspace) if splits > 1 else 0, sink=int(sink is not None), sink_w=ptr(sink),
+                        softcap=float(softcap))
     call_dense("i64h_latent_attn", _ref(d), _stream())
     return out
 
@@ -156,8 +163,9 @@ def _rows_ok(name: str, n: int, *tensors) -> None:
 
 def embed_bigram(ids: torch.Tensor, positions: torch.Tensor, slot_ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, *,
                  bigram: Optional[torch.Tensor] = None, buckets: int = 0, mul_prev: int = 0, mul_cur: int = 0,
-                 prev_token: Optional[torch.Tensor] = None, pos_table: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """See i64h_embed_bigram.  out fp32 [copies, n, W] (or [n, W]); prev_token int64 [slots], read and updated; pos_table bf16 [positions, W]."""
+                 prev_token: Optional[torch.Tensor] = None, pos_table: Optional[torch.Tensor] = None, scale: float = 1.0) -> torch.Tensor:
+    """See i64h_embed_bigram.  out fp32 [copies, n, W] (or [n, W]); prev_token int64 [slots], read and updated; pos_table bf16 [positions, W];
+    scale multiplies the token row."""
     _chk(ids, torch.int64, "ids"), _chk(positions, torch.int32, "positions"), _chk(slot_ids, torch.int32, "slot_ids")
     _chk(table, torch.bfloat16, "table"), _chk(out, torch.float32, "out")
     n = ids.numel()
@@ -176,7 +184,8 @@ def embed_bigram(ids: torch.Tensor, positions: torch.Tensor, slot_ids: torch.Ten
             raise _lib.I64HError(f"embed_bigram: position table {tuple(pos_table.shape)} for width {W}")
     d = _lib.EmbedBigram(ids=ptr(ids), positions=ptr(positions), slot_ids=ptr(slot_ids), table=ptr(table), V=V, W=W, bigram=ptr(bigram),
                          buckets=int(buckets), mul_prev=int(mul_prev), mul_cur=int(mul_cur), prev_token=ptr(prev_token), out=ptr(out),
-                         copies=max(1, copies), n=n, pos_table=ptr(pos_table), pos_rows=pos_table.shape[0] if pos_table is not None else 0)
+                         copies=max(1, copies), n=n, pos_table=ptr(pos_table), pos_rows=pos_table.shape[0] if pos_table is not None else 0,
+                         scale=float(scale))
     call_dense("i64h_embed_bigram", _ref(d), _stream())
     return out
 
@@ -184,11 +193,14 @@ def embed_bigram(ids: torch.Tensor, positions: torch.Tensor, slot_ids: torch.Ten
 def streams_step(streams: torch.Tensor, *, y: Optional[torch.Tensor] = None, y2: Optional[torch.Tensor] = None, yn_w: Optional[torch.Tensor] = None,
                  y2n_w: Optional[torch.Tensor] = None, y_eps: float = 0.0, mix: Optional[torch.Tensor] = None, out_w: Optional[torch.Tensor] = None,
                  in_w: Optional[torch.Tensor] = None, norm_w: Optional[torch.Tensor] = None, eps: float = 0.0, h: Optional[torch.Tensor] = None,
-                 rows: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
-    """See i64h_streams_step.  streams fp32 [S, n, W], updated in place when y is given; h fp32 [n, W] (or [rows, W])."""
+                 rows: Optional[torch.Tensor] = None, post_w: Optional[torch.Tensor] = None, post_center: bool = False,
+                 h_center: bool = False) -> Optional[torch.Tensor]:
+    """See i64h_streams_step.  streams fp32 [S, n, W], updated in place when y is given; h fp32 [n, W] (or [rows, W]).  post_w fp32 [W]: a
+    norm over the result as a whole (centred with post_center) before it is added; h_center: the read's norm is centred."""
     _chk(streams, torch.float32, "streams")
     S, n, W = streams.shape
-    for t, name in ((y, "y"), (y2, "y2"), (yn_w, "yn_w"), (y2n_w, "y2n_w"), (mix, "mix"), (out_w, "out_w"), (in_w, "in_w"), (norm_w, "norm_w"), (h, "h")):
+    for t, name in ((y, "y"), (y2, "y2"), (yn_w, "yn_w"), (y2n_w, "y2n_w"), (mix, "mix"), (out_w, "out_w"), (in_w, "in_w"), (norm_w, "norm_w"), (h, "h"),
+                    (post_w, "post_w")):
         if t is not None:
             _chk(t, torch.float32, name)
     for t, name in ((y, "y"), (y2, "y2")):
@@ -196,7 +208,7 @@ def streams_step(streams: torch.Tensor, *, y: Optional[torch.Tensor] = None, y2:
             raise _lib.I64HError(f"streams_step: {name} is not [n, W]")
     if (mix is not None and mix.numel() != S * S) or (out_w is not None and out_w.numel() != S) or (in_w is not None and in_w.numel() != S):
         raise _lib.I64HError("streams_step: stream weights do not fit the number of streams")
-    if (yn_w is not None and yn_w.numel() != W) or (y2n_w is not None and y2n_w.numel() != W):
+    if (yn_w is not None and yn_w.numel() != W) or (y2n_w is not None and y2n_w.numel() != W) or (post_w is not None and post_w.numel() != W):
         raise _lib.I64HError("streams_step: result norm weights are not [W]")
     m_rows = n
     if rows is not None:
@@ -206,7 +218,7 @@ def streams_step(streams: torch.Tensor, *, y: Optional[torch.Tensor] = None, y2:
         raise _lib.I64HError("streams_step: h smaller than the rows it receives")
     d = _lib.Streams(streams=ptr(streams), S=S, n=n, W=W, y=ptr(y), ldy=W, y2=ptr(y2), ldy2=W, yn_w=ptr(yn_w), y2n_w=ptr(y2n_w), y_eps=float(y_eps),
                      mix=ptr(mix), out_w=ptr(out_w), in_w=ptr(in_w), norm_w=ptr(norm_w), norm_w_len=norm_w.numel() if norm_w is not None else 0,
-                     eps=float(eps), h=ptr(h), rows=ptr(rows), m_rows=m_rows)
+                     eps=float(eps), h=ptr(h), rows=ptr(rows), m_rows=m_rows, post_w=ptr(post_w), post_center=int(bool(post_center)), h_center=int(bool(h_center)))
     call_dense("i64h_streams_step", _ref(d), _stream())
     return h
 
@@ -259,10 +271,14 @@ def ssm_scan(xbc: torch.Tensor, dt: torch.Tensor, *, dt_off: int, lddt: int, dt_
 
 
 def gate_norm(y: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, groups: int, eps: float, z: Optional[torch.Tensor] = None, z_off: int = 0,
-              ldz: int = 0, n: Optional[int] = None) -> torch.Tensor:
-    """out = rms_groups(y * silu(z)) * w: see i64h_gate_norm.  y, out fp32 [n, width]; z the columns [z_off, + width) of a matrix of row stride ldz."""
+              ldz: int = 0, n: Optional[int] = None, gate_after: bool = False, width: Optional[int] = None) -> torch.Tensor:
+    """out = rms_groups(y * silu(z)) * w: see i64h_gate_norm.  y, out fp32 [n, width]; z the columns [z_off, + width) of a matrix of row stride ldz.
+    gate_after: out = rms_groups(y) * w * silu(z).  width (default: w's length): the row's width, w then repeats over it."""
     _chk(y, torch.float32, "y"), _chk(w, torch.float32, "w"), _chk(out, torch.float32, "out")
-    width = w.numel()
+    w_len = w.numel()
+    width = int(width if width is not None else w_len)
+    if width % w_len:
+        raise _lib.I64HError("gate_norm: the weights do not repeat evenly over the row")
     rows = int(n if n is not None else y.numel() // width)
     if y.numel() < rows * width or out.numel() < rows * width:
         raise _lib.I64HError("gate_norm: operand smaller than the launch reads or writes")
@@ -271,7 +287,7 @@ def gate_norm(y: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, groups: in
         if z.numel() < (rows - 1) * ldz + z_off + width:
             raise _lib.I64HError("gate_norm: gate smaller than the launch reads")
     d = _lib.GateNorm(y=ptr(y), ldy=width, z=(ptr(z) + 4 * z_off) if z is not None else 0, ldz=ldz, w=ptr(w), width=width, groups=groups, eps=float(eps),
-                      out=ptr(out), ldo=width, n=rows)
+                      out=ptr(out), ldo=width, n=rows, gate_after=int(bool(gate_after)), w_len=w_len if w_len != width else 0)
     call_dense("i64h_gate_norm", _ref(d), _stream())
     return out
 
@@ -315,7 +331,7 @@ def kattn_prep(p: torch.Tensor, *, q_off: int, k_off: int, heads: int, kv_heads:
 
 def kattn(q: torch.Tensor, cache: torch.Tensor, kscale: torch.Tensor, block_table: torch.Tensor, slot_ids: torch.Tensor, positions: torch.Tensor, *,
           chunk: int, bias: Optional[torch.Tensor], sink: bool, heads: int, kv_heads: int, dim: int, out: torch.Tensor, n: Optional[int] = None,
-          mode: int = 0, splits: int = 1, workspace: Optional[torch.Tensor] = None, vdim: int = 0) -> torch.Tensor:
+          mode: int = 0, splits: int = 1, workspace: Optional[torch.Tensor] = None, vdim: int = 0, softcap: float = 0.0) -> torch.Tensor:
     """See i64h_kattn.  q, out fp32 [n, heads * dim]; bias fp32 [distances, heads].  vdim > 0: separate values - the cache rows are
     [kv_heads, vdim + dim], q fp32 [n, heads, vdim + dim], out fp32 [n, heads * vdim], kscale may be None."""
     _chk(q, torch.float32, "q"), _chk(out, torch.float32, "out"), _chk(cache, None, "cache")
@@ -343,7 +359,7 @@ def kattn(q: torch.Tensor, cache: torch.Tensor, kscale: torch.Tensor, block_tabl
                    max_blocks_per_seq=block_table.shape[1], block_size=cache.shape[-2], slot_ids=ptr(slot_ids), positions=ptr(positions), chunk=int(chunk),
                    bias=ptr(bias), bias_rows=bias.shape[0] if bias is not None else 0, sink=int(bool(sink)), out=ptr(out), n=rows, heads=heads,
                    kv_heads=kv_heads, dim=dim, mode=int(mode), splits=int(splits) if splits > 1 else 1, workspace=ptr(workspace) if splits > 1 else 0,
-                   vdim=int(vdim))
+                   vdim=int(vdim), softcap=float(softcap))
     call_dense("i64h_kattn", _ref(d), _stream())
     return out
 
@@ -373,6 +389,92 @@ def kv_prep(p: torch.Tensor, *, q_off: int, k_off: int, v_off: int, heads: int, 
                     block_size=cache.shape[-2] if cache is not None else int(block_size), cache=ptr(cache),
                     cache_dtype=CACHE_DTYPE_CODE[cache.dtype] if cache is not None else 0, Q=ptr(q), n=rows)
     call_dense("i64h_kv_prep", _ref(d), _stream())
+
+
+def rot_prep(p: torch.Tensor, *, q_off: int, k_off: int, v_off: int, heads: int, kv_heads: int, dim: int, vdim: int, q_norm_w: Optional[torch.Tensor],
+             k_norm_w: Optional[torch.Tensor], eps: float, rot_dims: int, interleaved: bool, inv_freq: Optional[torch.Tensor], rot_mult: float,
+             head_norm: bool, v_freq: Optional[torch.Tensor], scale: float, positions: torch.Tensor, slot_ids: torch.Tensor, block_table: torch.Tensor,
+             cache: torch.Tensor, q: torch.Tensor, n: Optional[int] = None) -> None:
+    """See i64h_rot_prep.  cache [blocks, block, kv_heads * (vdim + dim)] fp32 / bf16; q fp32 [n, heads, vdim + dim]; inv_freq fp32 [rot_dims / 2];
+    v_freq fp32 [vdim / 2] or None."""
+    _chk(p, torch.float32, "p"), _chk(q, torch.float32, "q"), _chk(cache, None, "cache")
+    _chk(positions, torch.int32, "positions"), _chk(slot_ids, torch.int32, "slot_ids"), _chk(block_table, torch.int32, "block_table")
+    rows = int(n if n is not None else positions.numel())
+    _rows_ok("rot_prep", rows, positions, slot_ids)
+    gs = vdim + dim
+    if q.numel() < rows * heads * gs or max(q_off + heads * dim, k_off + kv_heads * dim, v_off + kv_heads * vdim) > p.shape[-1] or p.numel() < rows * p.shape[-1] or \
+            cache.shape[-1] != kv_heads * gs:
+        raise _lib.I64HError("rot_prep: shapes do not fit the sizes")
+    for t, name, size in ((q_norm_w, "q_norm_w", heads * dim), (k_norm_w, "k_norm_w", kv_heads * dim), (inv_freq, "inv_freq", rot_dims // 2), (v_freq, "v_freq", vdim // 2)):
+        if t is not None:
+            _chk(t, torch.float32, name)
+            if t.numel() < size:
+                raise _lib.I64HError(f"rot_prep: {name} has {t.numel()} values, {size} needed")
+    if rot_dims and inv_freq is None:
+        raise _lib.I64HError("rot_prep: rotated dimensions without frequencies")
+    d = _lib.RotPrep(P=ptr(p), ldp=p.shape[-1], q_off=q_off, k_off=k_off, v_off=v_off, heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, q_norm_w=ptr(q_norm_w),
+                     k_norm_w=ptr(k_norm_w), eps=float(eps), rot_dims=int(rot_dims), interleaved=int(bool(interleaved)), inv_freq=ptr(inv_freq), rot_mult=float(rot_mult),
+                     head_norm=int(bool(head_norm)), v_freq=ptr(v_freq), scale=float(scale), positions=ptr(positions), slot_ids=ptr(slot_ids),
+                     block_table=ptr(block_table), max_blocks_per_seq=block_table.shape[1], block_size=cache.shape[-2], cache=ptr(cache),
+                     cache_dtype=CACHE_DTYPE_CODE[cache.dtype], Q=ptr(q), n=rows)
+    call_dense("i64h_rot_prep", _ref(d), _stream())
+
+
+def rot_post(o: torch.Tensor, *, heads: int, vdim: int, interleaved: bool, v_freq: Optional[torch.Tensor], positions: torch.Tensor,
+             gate: Optional[torch.Tensor] = None, gate_off: int = 0, ldg: int = 0, n: Optional[int] = None) -> torch.Tensor:
+    """See i64h_rot_post: o fp32 [n, heads, vdim] turned back by its row's position and gated per head, in place.  gate: the columns
+    [gate_off, + heads) of a matrix of row stride ldg."""
+    _chk(o, torch.float32, "o"), _chk(positions, torch.int32, "positions")
+    rows = int(n if n is not None else positions.numel())
+    _rows_ok("rot_post", rows, positions)
+    if o.numel() < rows * heads * vdim:
+        raise _lib.I64HError("rot_post: the output rows do not fit the sizes")
+    if v_freq is not None:
+        _chk(v_freq, torch.float32, "v_freq")
+        if v_freq.numel() < vdim // 2:
+            raise _lib.I64HError("rot_post: too few frequencies")
+    if gate is not None:
+        _chk(gate, torch.float32, "gate")
+        if gate.numel() < (rows - 1) * ldg + gate_off + heads:
+            raise _lib.I64HError("rot_post: gate smaller than the launch reads")
+    d = _lib.RotPost(O=ptr(o), heads=heads, vdim=vdim, interleaved=int(bool(interleaved)), v_freq=ptr(v_freq), positions=ptr(positions),
+                     gate=(ptr(gate) + 4 * gate_off) if gate is not None else 0, ldg=int(ldg), n=rows)
+    call_dense("i64h_rot_post", _ref(d), _stream())
+    return o
+
+
+def _gdn_args(x: torch.Tensor, g: torch.Tensor, *, q_off: int, k_off: int, v_off: int, heads: int, kv_heads: int, dim: int, vdim: int, n: int, **rest) -> "_lib.Gdn":
+    _chk(x, torch.float32, "x"), _chk(g, torch.float32, "g")
+    ld = x.shape[-1]
+    if max(q_off, k_off) + kv_heads * dim > ld or v_off + heads * vdim > ld or x.numel() < n * ld or g.numel() < n * 2 * heads:
+        raise _lib.I64HError("gdn: columns outside the rows, or too few gate rows")
+    return _lib.Gdn(X=ptr(x), ldx=ld, q_off=q_off, k_off=k_off, v_off=v_off, heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, G=ptr(g), n=n, **rest)
+
+
+def gdn_gates(x: torch.Tensor, g: torch.Tensor, raw: torch.Tensor, *, q_off: int, k_off: int, v_off: int, heads: int, kv_heads: int, dim: int, vdim: int,
+              b_off: int, a_off: int, a_log: torch.Tensor, dt_bias: torch.Tensor, unit_eps: float, q_scale: float, n: int) -> None:
+    """See i64h_gdn_gates: unit-vector queries and keys in place on x fp32 [n, ldx]; g fp32 [n, 2 * heads] receives write strength and decay from
+    the columns b_off / a_off of raw fp32 [n, ldr]."""
+    _chk(raw, torch.float32, "raw"), _chk(a_log, torch.float32, "a_log"), _chk(dt_bias, torch.float32, "dt_bias")
+    if max(b_off, a_off) + heads > raw.shape[-1] or raw.numel() < n * raw.shape[-1] or min(a_log.numel(), dt_bias.numel()) < heads:
+        raise _lib.I64HError("gdn_gates: shapes do not fit the sizes")
+    d = _gdn_args(x, g, q_off=q_off, k_off=k_off, v_off=v_off, heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, n=n, R=ptr(raw), ldr=raw.shape[-1],
+                  b_off=b_off, a_off=a_off, A_log=ptr(a_log), dt_bias=ptr(dt_bias), unit_eps=float(unit_eps), q_scale=float(q_scale))
+    call_dense("i64h_gdn_gates", _ref(d), _stream())
+
+
+def gdn_scan(x: torch.Tensor, g: torch.Tensor, *, q_off: int, k_off: int, v_off: int, heads: int, kv_heads: int, dim: int, vdim: int, seg_start: torch.Tensor,
+             nseg: int, positions: torch.Tensor, slot_ids: torch.Tensor, state: torch.Tensor, out: torch.Tensor, n: int) -> torch.Tensor:
+    """See i64h_gdn_scan.  state fp32 [slots, heads, vdim, dim]; out fp32 [n, heads * vdim]."""
+    _chk(state, torch.float32, "state"), _chk(out, torch.float32, "out")
+    _chk(seg_start, torch.int32, "seg_start"), _chk(positions, torch.int32, "positions"), _chk(slot_ids, torch.int32, "slot_ids")
+    _rows_ok("gdn_scan", n, positions, slot_ids)
+    if tuple(state.shape[1:]) != (heads, vdim, dim) or out.numel() < n * heads * vdim or seg_start.numel() < nseg + 1:
+        raise _lib.I64HError("gdn_scan: shapes do not fit the sizes")
+    d = _gdn_args(x, g, q_off=q_off, k_off=k_off, v_off=v_off, heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, n=n, seg_start=ptr(seg_start), nseg=nseg,
+                  positions=ptr(positions), slot_ids=ptr(slot_ids), state=ptr(state), out=ptr(out), ldo=heads * vdim)
+    call_dense("i64h_gdn_scan", _ref(d), _stream())
+    return out
 
 
 def _gla_args(p: torch.Tensor, *, q_off: int, f_off: int, v_off: int, heads: int, dim: int, vdim: int, k_off: int = -1, lower: Optional[torch.Tensor] = None,

@@ -59,6 +59,18 @@ def _load_zabutar(config: dict, tensors, *, device, dtype, max_seqs, max_tokens,
     return ZabutarModel(cfg, tensors, device=device, dtype=dtype, max_seqs=max_seqs, num_kv_blocks=blocks, kv_block=kv_block)
 
 
+def _load_fukatar(config: dict, tensors, *, device, dtype, max_seqs, max_tokens, kv_block=16, **_):
+    from .config import FukatarConfig
+    from .fukatar import FukatarModel
+    config = dict(config)
+    for key, axis in (("vocab", 0), ("width", 1)):      # sizes that the file may leave to the tensors' shapes
+        if key not in config and "embed" in tensors:
+            config[key] = int(tensors["embed"].shape[axis])
+    cfg = FukatarConfig.from_dict(config)
+    blocks = max(1, (int(max_tokens) + kv_block - 1) // kv_block)
+    return FukatarModel(cfg, tensors, device=device, dtype=dtype, max_seqs=max_seqs, num_kv_blocks=blocks, kv_block=kv_block)
+
+
 def _load_complexity_deep(config: dict, tensors, *, device, dtype, max_seqs, max_tokens, quant="int8", **_):
     import torch
     from .checkpoint import config_from_dict, native_to_weights
@@ -72,6 +84,7 @@ def _load_complexity_deep(config: dict, tensors, *, device, dtype, max_seqs, max
 register("Morilorn", _load_morilorn)
 register("Dogalorn", _load_dogalorn)
 register("Zabutar", _load_zabutar)
+register("Fukatar", _load_fukatar)
 register("complexity-deep", _load_complexity_deep)
 register("ComplexityDeepModel", _load_complexity_deep)
 
