@@ -60,7 +60,7 @@ def parse():
                          "(e4m3fn weights per output channel, e4m3fn activations per token) on the fp8 matrix cores")
     ap.add_argument("--no-replica-leg", action="store_true",
                     help="N > 1: skip the second, labelled measurement of independent replicas (reported beside the expert-parallel value)")
-    ap.add_argument("--design", default="", choices=["", "morilorn", "dogalorn", "zabutar"],
+    ap.add_argument("--design", default="", choices=["", "morilorn", "dogalorn", "zabutar", "fukatar"],
                     help="instead of the headline workload: prefill / decode throughput of another registered design at real layer sizes beside "
                          "the closest existing model, and its kernels against their rooflines (vllm_i64_amd/bench_designs.py)")
     ap.add_argument("--design-sizes", default="", help="--design: sizes to run, with commas between them (default: all)")

@@ -1,0 +1,631 @@
+"""The Fukatar design on the GPU against the CPU oracle (oracle/fukatar_ref.py): every mechanism alone, then whole models of several
+small shapes under every way of cutting, batching, paging and slotting their sequences, through the engine and the command line.
+Weights are random and bf16-representable; where random weights would hide a fault (a far key among many, a sink, a state that has to
+last) the inputs are made so that it shows.  Mechanism tests feed the kernels projection rows directly: the oracle gets the same rows
+as its input and selector matrices as its projections."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+from oracle import fukatar_ref as R
+from tests.fukatar_shapes import SHAPES, config_of, make_weights, tokens
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+# rms over the vocabulary of the logit difference / rms of the logits.  bfloat16: the 2^-9 input rounding of every matrix product,
+# carried on by the recurrence and blown up where a sublayer's result is small before its norm, gives a few percent; a wrong
+# mechanism gives 50 % and more at every position.
+TOL = {"float32": 3e-5, "bfloat16": 8e-2}
+F64 = torch.float64
+
+
+@pytest.fixture(scope="module")
+def dev():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    return torch.device("cuda:0")
+
+
+def row_err(got, want):
+    got, want = torch.as_tensor(got, dtype=F64).cpu(), torch.as_tensor(want, dtype=F64).cpu()
+    d = got - want
+    d = d - d.mean(-1, keepdim=True)
+    return d.pow(2).mean(-1).sqrt() / want.pow(2).mean(-1).sqrt().clamp_min(1e-9)
+
+
+def agrees(got, want, dtype):
+    e = row_err(got, want).flatten()
+    if dtype == "float32":
+        return float(e.max()) < TOL[dtype]
+    return int((e >= TOL[dtype]).sum()) <= max(1, e.numel() // 30) and float(e.max()) < 4 * TOL[dtype]
+
+
+def same_to_rounding(got, want, dtype):
+    """Two runs of the same model that differ in how the sequence was cut, batched or placed: only the order of sums may differ (in
+    bfloat16 a last bit of a sum can move a rounded input of the next product by one step, hence the looser bound)."""
+    e = row_err(got, want).flatten()
+    tol = 2e-5 if dtype == "float32" else 2e-2
+    return float(e.median()) < tol and float((e < 5 * tol).double().mean()) >= 0.9
+
+
+def close(got, want, tol=2e-5):
+    got, want = torch.as_tensor(got, dtype=F64).cpu(), torch.as_tensor(want, dtype=F64).cpu()
+    return float((got - want).abs().max() / want.abs().max().clamp_min(1e-9)) <= tol
+
+
+def make_model(name, dtype, dev, max_tokens=512, max_seqs=4, seed=0, block=16):
+    from vllm_i64_amd.config import FukatarConfig
+    from vllm_i64_amd.fukatar import FukatarModel
+    return FukatarModel(FukatarConfig.from_dict(config_of(name)), make_weights(name, seed), device=dev, dtype=dtype, max_seqs=max_seqs,
+                        num_kv_blocks=(max_tokens + block - 1) // block, kv_block=block)
+
+
+def oracle_logits(name, toks, seed=0, layers=None):
+    return R.forward(config_of(name), make_weights(name, seed), toks, layers)
+
+
+def whole_prompt(model, name, toks, dtype, slot=0, layers_too=False):
+    dev, n = model.device, len(toks)
+    model.kv.reserve(slot, n)
+    rec = {}
+    got = model.forward(torch.tensor(toks, dtype=torch.int64, device=dev), torch.arange(n, dtype=torch.int32, device=dev),
+                        torch.full((n,), slot, dtype=torch.int32, device=dev), record=rec, tokens_per_seq=[n]).cpu().clone()
+    model.kv.free(slot)
+    layers = []
+    want = oracle_logits(name, toks, layers=layers)
+    if layers_too:
+        for i, x in enumerate(layers):
+            assert agrees(rec[f"l{i}.x"], x, dtype), f"residual after layer {i}"
+    assert agrees(got, want, dtype)
+    return got
+
+
+def replay(engine, requests, schedule):
+    """schedule: steps of [(id, count)]; every position's logits are asked for.  Returns id -> [T, V] (CPU)."""
+    at = {i: 0 for i in requests}
+    got = {i: [] for i in requests}
+    for step in schedule:
+        entries, end = [], []
+        for i, count in step:
+            lo, hi = at[i], at[i] + count
+            entries.append((i, requests[i][lo:hi], list(range(count))))
+            at[i] = hi
+            if hi == len(requests[i]):
+                end.append(i)
+        lg = engine.step(entries, end=end).cpu()
+        row = 0
+        for i, count in step:
+            got[i].append(lg[row:row + count].clone())
+            row += count
+    return {i: torch.cat(v) for i, v in got.items() if v}
+
+
+class Rows:
+    """Rows of a step for op-level calls: sequences of (slot, first position, count) laid out one after the other."""
+
+    def __init__(self, dev, runs):
+        self.slots = torch.tensor([s for s, p, c in runs for _ in range(c)], dtype=torch.int32, device=dev)
+        self.pos = torch.tensor([p + j for s, p, c in runs for j in range(c)], dtype=torch.int32, device=dev)
+        st = [0]
+        for s, p, c in runs:
+            st.append(st[-1] + c)
+        self.seg = torch.tensor(st, dtype=torch.int32, device=dev)
+        self.nseg, self.n = len(runs), st[-1]
+
+
+def cuts_of(T, sizes):
+    out, at, i = [], 0, 0
+    while at < T:
+        c = min(sizes[i % len(sizes)], T - at)
+        out.append((at, c))
+        at += c
+        i += 1
+    return out
+
+
+def steps_of(lens, cut_sizes):
+    """Steps of [(slot, first position, count)] that run the sequences side by side under the same cut sizes."""
+    cuts = {s: cuts_of(T, cut_sizes) for s, T in lens.items()}
+    return [[(s, *cuts[s][k]) for s in lens if k < len(cuts[s])] for k in range(max(len(c) for c in cuts.values()))]
+
+
+def pages(dev, slots, blocks_per_seq, block, seed):
+    """A block table whose pages lie scattered over the pool."""
+    perm = torch.randperm(slots * blocks_per_seq, generator=torch.Generator().manual_seed(seed)).to(torch.int32)
+    return perm.reshape(slots, blocks_per_seq).to(dev)
+
+
+def selectors(widths):
+    """name -> the rows of an identity that pick that part of a concatenated row."""
+    total, out, at = sum(widths.values()), {}, 0
+    for k, n in widths.items():
+        out[k] = torch.eye(total, dtype=F64)[at:at + n]
+        at += n
+    return out, total
+
+
+# =================================================== mechanisms alone =============================================================
+@pytest.mark.parametrize("M", [1, 5, 40, 150])
+@pytest.mark.parametrize("exact", [False, True])
+def test_linear_squared_relu_epilogue(dev, M, exact):
+    from vllm_i64_amd import ops_dense as D
+    g = torch.Generator().manual_seed(M)
+    K, N = 72, 52
+    a = torch.randn(M, K, generator=g)
+    if not exact:
+        a = a.to(torch.bfloat16).float()
+    w = (torch.randn(N, K, generator=g) * K ** -0.5).to(torch.bfloat16)
+    out = torch.empty(M, N, device=dev)
+    D.linear(a.to(dev), w.to(dev), out, exact=exact, epilogue=D.EPI_RELU_SQ)
+    want = torch.relu(a.double() @ w.double().T).pow(2)
+    assert float((want == 0).double().mean()) > 0.2 and close(out, want, 1e-5)
+
+
+@pytest.mark.parametrize("cut_sizes", [[50], [1], [2, 7, 1]])
+def test_embedding_scale_and_bigram_rows_under_cuts(dev, cut_sizes):
+    """The previous token crosses the cuts through the slot's state, which is stale at the start; the first token takes the last row."""
+    from vllm_i64_amd import ops_dense as D
+    g = torch.Generator().manual_seed(3)
+    V, W, e = 37, 24, {"scale": 2.5, "bigram": {"buckets": 11, "mul_prev": 1000003, "mul_cur": 17}}
+    Wt = {"embed": torch.randn(V, W, generator=g).to(torch.bfloat16), "bigram": torch.randn(12, W, generator=g).to(torch.bfloat16)}
+    toks = {1: torch.randint(0, V, (23,), generator=g).tolist(), 0: torch.randint(0, V, (9,), generator=g).tolist()}
+    want = {s: R.embedding({k: v.double() for k, v in Wt.items()}, e, t) for s, t in toks.items()}
+    prev = torch.full((2,), 5, dtype=torch.int64, device=dev)
+    got = {s: [] for s in toks}
+    for runs in steps_of({s: len(t) for s, t in toks.items()}, cut_sizes):
+        r = Rows(dev, runs)
+        ids = torch.tensor([t for s, p, c in runs for t in toks[s][p:p + c]], dtype=torch.int64, device=dev)
+        out = torch.empty(1, r.n, W, device=dev)
+        D.embed_bigram(ids, r.pos, r.slots, Wt["embed"].to(dev), out, bigram=Wt["bigram"].to(dev), buckets=11, mul_prev=1000003, mul_cur=17, prev_token=prev, scale=2.5)
+        row = 0
+        for s, p, c in runs:
+            got[s].append(out[0, row:row + c].cpu())
+            row += c
+    for s in toks:
+        assert close(torch.cat(got[s]), want[s], 1e-6)
+
+
+@pytest.mark.parametrize("cut_sizes", [[40], [1], [2, 5, 1, 3], [600]])
+def test_token_shift_under_cuts(dev, cut_sizes):
+    """The blend with the row before as the two-tap added convolution the runner uses; slots with stale carried rows."""
+    from vllm_i64_amd import ops_dense as D
+    g = torch.Generator().manual_seed(len(cut_sizes))
+    W = 70
+    lens = {2: 37, 0: 9, 1: 640 if cut_sizes == [600] else 23}
+    s_w = torch.rand(W, generator=g)
+    x = {s: torch.randn(T, W, generator=g) for s, T in lens.items()}
+    want = {s: R.token_shift(s_w.double(), x[s].double()) for s in lens}
+    state = torch.full((3, 1, W), 9.0, device=dev)
+    w2 = torch.stack([s_w, -s_w], 1).contiguous().to(dev)
+    got = {s: [] for s in lens}
+    for runs in steps_of(lens, cut_sizes):
+        r = Rows(dev, runs)
+        rows = torch.cat([x[s][p:p + c] for s, p, c in runs]).to(dev).contiguous()
+        out = torch.empty(r.n, W, device=dev)
+        D.causal_conv(rows, off=0, channels=W, w=w2, bias=None, positions=r.pos, slot_ids=r.slots, state=state, out=out, n=r.n, added=True,
+                      single_rows=all(c == 1 for _, _, c in runs))
+        row = 0
+        for s, p, c in runs:
+            got[s].append(out[row:row + c].cpu())
+            row += c
+    for s in lens:
+        assert close(torch.cat(got[s]), want[s], 1e-5), s
+
+
+@pytest.mark.parametrize("W", [24, 300])
+def test_residual_takes_centred_norms_of_one_result_and_of_two(dev, W):
+    from vllm_i64_amd import ops_dense as D
+    g = torch.Generator().manual_seed(W)
+    n, eps = 7, 1e-5
+    x = torch.randn(1, n, W, generator=g)
+    y, y2 = torch.randn(n, W, generator=g) * 3 + 2.0, torch.randn(n, W, generator=g) * 0.2 - 1.0      # (means that matter)
+    w, wl, wr, wf = (torch.rand(W, generator=g) + 0.5 for _ in range(4))
+    ones = torch.ones(1, device=dev)
+    xs = x.to(dev).clone()
+    D.streams_step(xs, y=y.to(dev), y_eps=eps, out_w=ones, post_w=w.to(dev), post_center=True)
+    want = x[0].double() + R.layer_norm(y.double(), w.double(), eps)
+    assert close(xs[0], want, 1e-6)
+    D.streams_step(xs, y=y.to(dev), y2=y2.to(dev), yn_w=wl.to(dev), y2n_w=wr.to(dev), y_eps=eps, out_w=ones, post_w=w.to(dev), post_center=True)
+    both = 0.5 * (R.rms(y.double(), eps) * wl.double() + R.rms(y2.double(), eps) * wr.double())
+    want = want + R.layer_norm(both, w.double(), eps)
+    assert close(xs[0], want, 1e-6)
+    rows = torch.tensor([5, 0, 5, 2], dtype=torch.int32, device=dev)
+    h = torch.empty(4, W, device=dev)
+    D.streams_step(xs, norm_w=wf.to(dev), eps=eps, h=h, rows=rows, h_center=True)
+    assert close(h, R.layer_norm(want[rows.cpu().long()], wf.double(), eps), 1e-5)
+
+
+def _rotary_case(H, G, d, dv, dims, scaling, cap, flavour):
+    """Config entry, oracle function and kernel options of the two rotated attentions."""
+    m = {"heads": H, "kv_heads": G, "dim": d, "vdim": dv, "scale": 0.37, "softcap": cap, "rot": {"base": 300.0, "dims": dims}}
+    if scaling:
+        m["rot"]["scaling"] = dict(zip(("factor", "original", "fast", "slow"), scaling))
+    return m, (R.rotary_attention if flavour == "gated" else R.unit_norm_attention)
+
+
+def _run_rotary(dev, m, flavour, rows_of, lens, cut_sizes, cache_dtype, block, eps, norm_w=None, mode=None):
+    """rows_of: slot -> [T, q | k | v | g] projection rows.  The kernels under cuts over scattered pages; returns slot -> [T, H * dv]."""
+    from vllm_i64_amd import ops_dense as D
+    from vllm_i64_amd.config import RotaryConfig
+    H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+    gated = flavour == "gated"
+    rc = RotaryConfig.from_dict(m["rot"])
+    fr, mult = rc.frequencies()
+    inv = torch.tensor(fr, dtype=F64).float().to(dev) if rc.dims else None
+    vf = torch.tensor([rc.base ** (-2.0 * i / dv) for i in range(dv // 2)], dtype=F64).float().to(dev) if gated else None
+    gs, nq, nk, nv = dv + d, H * d, G * d, G * dv
+    ld = nq + nk + nv + H
+    per_seq = (max(lens.values()) + block - 1) // block
+    bt = pages(dev, 3, per_seq, block, 5)
+    cache = torch.full((3 * per_seq, block, G * gs), 7.0, dtype=cache_dtype, device=dev)
+    got = {s: [] for s in lens}
+    for runs in steps_of(lens, cut_sizes):
+        r = Rows(dev, runs)
+        P = torch.cat([rows_of[s][p:p + c] for s, p, c in runs]).float().to(dev).contiguous()
+        Q = torch.empty(r.n, H * gs, device=dev)
+        D.rot_prep(P, q_off=0, k_off=nq, v_off=nq + nk, heads=H, kv_heads=G, dim=d, vdim=dv, q_norm_w=norm_w[0].float().to(dev) if gated else None,
+                   k_norm_w=norm_w[1].float().to(dev) if gated else None, eps=eps, rot_dims=rc.dims, interleaved=not gated, inv_freq=inv, rot_mult=mult,
+                   head_norm=not gated, v_freq=vf, scale=m["scale"], positions=r.pos, slot_ids=r.slots, block_table=bt, cache=cache, q=Q, n=r.n)
+        O = torch.empty(r.n, H * dv, device=dev)
+        one = all(c == 1 for _, _, c in runs)
+        D.kattn(Q, cache, None, bt, r.slots, r.pos, chunk=0, bias=None, sink=False, heads=H, kv_heads=G, dim=d, vdim=dv, out=O, n=r.n,
+                mode=mode if mode is not None else (2 if one else 3), softcap=m["softcap"] or 0.0)
+        if gated:
+            D.rot_post(O, heads=H, vdim=dv, interleaved=False, v_freq=vf, positions=r.pos, gate=P, gate_off=nq + nk + nv, ldg=ld, n=r.n)
+        row = 0
+        for s, p, c in runs:
+            got[s].append(O[row:row + c].cpu())
+            row += c
+    return {s: torch.cat(v) for s, v in got.items()}
+
+
+def _rotary_oracle(m, fn, rows, eps, norm_w):
+    H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+    sel, _ = selectors({"q": H * d, "k": G * d, "v": G * dv, "g": H})
+    W = {"x." + k: v for k, v in sel.items()}
+    W.update({"x.q.norm": norm_w[0].double(), "x.k.norm": norm_w[1].double(), "x.o": torch.eye(H * dv, dtype=F64)})
+    return fn(W, "x.", m, eps, rows.double())
+
+
+@pytest.mark.parametrize("flavour", ["gated", "unit"])
+@pytest.mark.parametrize("H,G,d,dv,dims", [(3, 3, 16, 16, 16), (6, 2, 10, 14, 6), (4, 1, 24, 40, 2), (2, 2, 130, 6, 64)])
+@pytest.mark.parametrize("block,cut_sizes", [(16, [300]), (4, [1]), (8, [2, 11, 1, 64])])
+def test_rotated_attention_in_32_bits(dev, flavour, H, G, d, dv, dims, block, cut_sizes):
+    g = torch.Generator().manual_seed(H * d + block)
+    m, fn = _rotary_case(H, G, d, dv, dims, (3.0, 48, 6.0, 0.5) if dims > 2 else None, 5.0, flavour)
+    lens = {2: 70, 0: 33, 1: 5}
+    ld = H * d + G * d + G * dv + H
+    rows = {s: torch.randn(T, ld, generator=g) for s, T in lens.items()}
+    nw = (torch.rand(H * d, generator=g) + 0.5, torch.rand(G * d, generator=g) + 0.5)
+    got = _run_rotary(dev, m, flavour, rows, lens, cut_sizes, torch.float32, block, 1e-5, nw)
+    for s in lens:
+        assert close(got[s], _rotary_oracle(m, fn, rows[s], 1e-5, nw), 2e-5), s
+
+
+@pytest.mark.parametrize("flavour", ["gated", "unit"])
+@pytest.mark.parametrize("H,G,d,dv,dims", [(3, 3, 16, 16, 8), (8, 2, 48, 32, 48), (34, 2, 32, 16, 30), (2, 1, 64, 256, 64), (4, 2, 40, 64, 12)])
+@pytest.mark.parametrize("block,cut_sizes", [(16, [200]), (4, [1]), (16, [2, 11, 1, 40])])
+def test_rotated_attention_matrix_core_form(dev, flavour, H, G, d, dv, dims, block, cut_sizes):
+    """The bf16 cache rounds keys and values after norm and rotation; scores, cap and softmax stay in 32 bits."""
+    g = torch.Generator().manual_seed(H * d + block)
+    m, fn = _rotary_case(H, G, d, dv, dims, (2.0, 64, 8.0, 1.0), 8.0, flavour)
+    lens = {2: 140, 0: 33, 1: 5}
+    ld = H * d + G * d + G * dv + H
+    rows = {s: torch.randn(T, ld, generator=g) for s, T in lens.items()}
+    nw = (torch.rand(H * d, generator=g) + 0.5, torch.rand(G * d, generator=g) + 0.5)
+    got = _run_rotary(dev, m, flavour, rows, lens, cut_sizes, torch.bfloat16, block, 1e-6, nw)
+    for s in lens:
+        assert close(got[s], _rotary_oracle(m, fn, rows[s], 1e-6, nw), 2.5e-2), s
+
+
+@pytest.mark.parametrize("flavour", ["gated", "unit"])
+@pytest.mark.parametrize("mode", ["prompt", "decode"])
+@pytest.mark.parametrize("cache_dtype,block,T", [(torch.float32, 16, 200), (torch.bfloat16, 8, 530)])
+def test_rotated_attention_one_key_stands_out(dev, flavour, mode, cache_dtype, block, T):
+    """One key alone lines up with the last query (along a dimension that is not rotated; every other key is orthogonal to it, so the
+    norms change nothing) - the first, one far back, those at page borders, the query's own: the head returns that key's value (with
+    rotated values: turned by its distance from the query), times the gate."""
+    H, G, d, dv = 2, 1, 16, 16
+    m, fn = _rotary_case(H, G, d, dv, 8, None, 30.0, flavour)
+    m["scale"] = 1.5
+    nw = (torch.ones(H * d), torch.ones(G * d))
+    g = torch.Generator().manual_seed(T)
+    ld = H * d + G * d + G * dv + H
+    for target in (0, 3, block - 1, block, T - 2 * block, T - 1):
+        rows = torch.zeros(T, ld)
+        v = torch.randn(T, dv, generator=g)
+        rows[:, H * d + G * d: H * d + G * d + dv] = v
+        rows[:, -H:] = 4.0
+        rows[:, H * d + 14] = 3.0
+        rows[target, H * d + 14], rows[target, H * d + 15] = 0.0, 3.0
+        rows[:, 15], rows[:, d + 15] = 1.0, 1.0
+        want = _rotary_oracle(m, fn, rows, 1e-6, nw)
+        lone = v[target].double().reshape(1, 1, dv)
+        if flavour == "gated":      # turned to its own position and back by the query's: by their distance, then the gate
+            lone = R.rotate(lone, torch.tensor([target - (T - 1)]), R.rotary_frequencies(300.0, dv)[0], dv, False) * torch.sigmoid(torch.tensor(4.0, dtype=F64))
+        assert close(want[-1].reshape(H, dv), lone.reshape(1, dv).expand(H, dv), 1e-4)      # (the premise)
+        cuts = [T] if mode == "prompt" else [T - 1, 1]
+        got = _run_rotary(dev, m, flavour, {1: rows}, {1: T}, cuts, cache_dtype, block, 1e-6, nw)
+        assert close(got[1][-1], want[-1], 2e-5 if cache_dtype == torch.float32 else 1e-2), target
+
+
+def test_rotated_attention_cap_decides(dev):
+    """Two keys whose scores differ by a wide margin but both lie far above the cap get nearly equal weights; without the cap one takes all."""
+    H, G, d, dv = 1, 1, 8, 8
+    m, fn = _rotary_case(H, G, d, dv, 0, None, 2.0, "gated")
+    m["scale"] = 10.0
+    rows = torch.zeros(2, H * d + G * d + G * dv + H)
+    rows[:, 0] = 1.0
+    rows[0, d], rows[1, d], rows[1, d + 1] = 1.0, 1.0, 1.0
+    rows[0, 2 * d], rows[1, 2 * d + 1] = 1.0, 1.0
+    rows[:, -1] = 20.0
+    nw = (torch.ones(d), torch.ones(d))
+    want = _rotary_oracle(m, fn, rows, 0.0, nw)
+    uncapped = _rotary_oracle(dict(m, softcap=None), fn, rows, 0.0, nw)
+    assert float((want[1] - uncapped[1]).abs().max()) > 0.3      # (the premise)
+    got = _run_rotary(dev, m, "gated", {0: rows}, {0: 2}, [2], torch.float32, 16, 0.0, nw)[0]
+    assert close(got, want, 1e-5)
+
+
+def _latent_run(dev, m, w, h, lens, cut_sizes, cache_dtype, block, eps, exact):
+    from vllm_i64_amd import ops_dense as D
+    H, d, dv, r = m["heads"], m["dim"], m["vdim"], m["kv_rank"]
+    per_seq = (max(lens.values()) + block - 1) // block
+    bt = pages(dev, 3, per_seq, block, 9)
+    cache = torch.full((3 * per_seq, block, r), 7.0, dtype=cache_dtype, device=dev)
+    uk_t = w["uk"].reshape(H, d, r).transpose(1, 2).contiguous().to(dev)
+    uv = w["uv"].reshape(H, dv, r).contiguous().to(dev)
+    N1 = H * d + r
+    got = {s: [] for s in lens}
+    for runs in steps_of(lens, cut_sizes):
+        rr = Rows(dev, runs)
+        P = torch.cat([h[s][p:p + c] for s, p, c in runs]).float().to(dev).contiguous()
+        Q = torch.empty(rr.n * H * r, device=dev)
+        D.latent_prep(P, q_off=0, dkv_off=H * d, heads=H, dim=d, rot_dim=0, kv_rank=r, rot_dims=0, c_norm_w=w["dkv.norm"].float().to(dev), eps=eps, inv_freq=None,
+                      positions=rr.pos, slot_ids=rr.slots, block_table=bt, block_size=block, cache=cache, q=Q, n=rr.n)
+        D.linear(P, uk_t, Q, m=rr.n, n=r, k=d, a_off=0, lda=N1, ldc=H * r, batch=H, a_batch=d, w_batch=r * d, c_batch=r, exact=exact)
+        olat = torch.empty(rr.n * H * r, device=dev)
+        one = all(c == 1 for _, _, c in runs)
+        D.latent_attn(Q, cache, bt, rr.slots, rr.pos, window=0, scale=m["scale"], heads=H, kv_rank=r, rot_dim=0, out=olat, n=rr.n, mode=2 if one else 3,
+                      sink=w["sink"].float().to(dev))
+        og = torch.empty(rr.n, H * dv, device=dev)
+        D.linear(olat, uv, og, m=rr.n, n=dv, k=r, lda=H * r, ldc=H * dv, batch=H, a_batch=r, w_batch=dv * r, c_batch=dv, exact=exact)
+        row = 0
+        for s, p, c in runs:
+            got[s].append(og[row:row + c].cpu())
+            row += c
+    return {s: torch.cat(v) for s, v in got.items()}
+
+
+@pytest.mark.parametrize("cache_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,d,dv,r", [(3, 10, 6, 18), (4, 32, 48, 64), (18, 16, 16, 32), (1, 24, 8, 128)])
+@pytest.mark.parametrize("block,cut_sizes", [(16, [200]), (4, [1]), (8, [2, 11, 1, 40])])
+def test_latent_attention_with_learned_sinks(dev, cache_dtype, H, d, dv, r, block, cut_sizes):
+    """Sinks from far below the scores (no effect) to far above them (the head returns next to nothing): leaving them out, scaling them
+    or counting them per key would show."""
+    g = torch.Generator().manual_seed(H + r + block)
+    m = {"heads": H, "dim": d, "vdim": dv, "kv_rank": r, "scale": 0.6 * d ** -0.5}
+    bf = lambda t: t.to(torch.bfloat16)
+    w = {"uk": bf(torch.randn(H * d, r, generator=g) * r ** -0.5), "uv": bf(torch.randn(H * dv, r, generator=g) * r ** -0.5), "dkv.norm": torch.rand(r, generator=g) + 0.5,
+         "sink": torch.linspace(-6.0, 6.0, H) if H > 1 else torch.tensor([1.5])}
+    lens = {2: 90, 0: 33, 1: 3}
+    h = {s: torch.randn(T, H * d + r, generator=g) * 2.0 for s, T in lens.items()}
+    exact = cache_dtype == torch.float32
+    if not exact:
+        h = {s: bf(v).float() for s, v in h.items()}
+    got = _latent_run(dev, m, w, h, lens, cut_sizes, cache_dtype, block, 1e-5, exact)
+    sel, _ = selectors({"q": H * d, "dkv": r})
+    W = {"x." + k: v for k, v in sel.items()}
+    W.update({"x.uk": w["uk"].double(), "x.uv": w["uv"].double(), "x.dkv.norm": w["dkv.norm"].double(), "x.sink": w["sink"].double(), "x.o": torch.eye(H * dv, dtype=F64)})
+    for s in lens:
+        want = R.latent_attention(W, "x.", m, 1e-5, h[s].double())
+        assert close(got[s], want, 2e-5 if exact else 3e-2), s
+    if H > 1:      # the sinks did something: the head with the highest sink returns much less than the one with the lowest
+        o = got[2].reshape(90, H, dv)
+        assert float(o[:, -1].abs().mean()) < 0.5 * float(o[:, 0].abs().mean())
+
+
+def _delta_run(dev, m, w, h, lens, cut_sizes, eps):
+    """h: slot -> [T, q | k | v | b | a | g] raw projections; convolution, gates, scan and the gated head norm through the kernels."""
+    from vllm_i64_amd import ops_dense as D
+    H, G, d, dv, taps = m["heads"], m["kv_heads"], m["dim"], m["vdim"], m["conv"]
+    rk, rv = G * d, H * dv
+    C, N1 = 2 * rk + rv, 2 * rk + 2 * rv + 2 * H
+    conv_w = torch.cat([w["q.conv"], w["k.conv"], w["v.conv"]], 0).float().contiguous().to(dev)
+    conv_state = torch.full((3, taps - 1, C), 9.0, device=dev) if taps > 1 else None
+    state = torch.full((3, H, dv, d), 9.0, device=dev)
+    got = {s: [] for s in lens}
+    for runs in steps_of(lens, cut_sizes):
+        r = Rows(dev, runs)
+        P = torch.cat([h[s][p:p + c] for s, p, c in runs]).float().to(dev).contiguous()
+        X = torch.empty(r.n, C, device=dev)
+        D.causal_conv(P, off=0, channels=C, w=conv_w, bias=None, positions=r.pos, slot_ids=r.slots, state=conv_state, out=X, n=r.n,
+                      single_rows=all(c == 1 for _, _, c in runs))
+        Gt = torch.empty(r.n, 2 * H, device=dev)
+        cols = dict(q_off=0, k_off=rk, v_off=2 * rk, heads=H, kv_heads=G, dim=d, vdim=dv, n=r.n)
+        D.gdn_gates(X, Gt, P, b_off=C, a_off=C + H, a_log=w["A_log"].float().to(dev), dt_bias=w["dt_bias"].float().to(dev), unit_eps=1e-6, q_scale=d ** -0.5, **cols)
+        O = torch.empty(r.n, rv, device=dev)
+        D.gdn_scan(X, Gt, seg_start=r.seg, nseg=r.nseg, positions=r.pos, slot_ids=r.slots, state=state, out=O, **cols)
+        On = torch.empty(r.n, rv, device=dev)
+        D.gate_norm(O, w["norm"].float().to(dev), On, groups=H, eps=eps, z=P, z_off=C + 2 * H, ldz=N1, n=r.n, gate_after=True, width=rv)
+        row = 0
+        for s, p, c in runs:
+            got[s].append(On[row:row + c].cpu())
+            row += c
+    return {s: torch.cat(v) for s, v in got.items()}
+
+
+def _delta_oracle(m, w, rows, eps):
+    H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+    sel, _ = selectors({"q": G * d, "k": G * d, "v": H * dv, "b": H, "a": H, "g": H * dv})
+    W = {"x." + k: v for k, v in sel.items()}
+    W.update({"x." + k: w[k].double() for k in ("q.conv", "k.conv", "v.conv", "A_log", "dt_bias", "norm")})
+    W["x.o"] = torch.eye(H * dv, dtype=F64)
+    return R.gated_delta(W, "x.", m, eps, rows.double())
+
+
+def _delta_weights(m, g, a_log=None):
+    H, G, d, dv, taps = m["heads"], m["kv_heads"], m["dim"], m["vdim"], m["conv"]
+    return {"q.conv": torch.randn(G * d, taps, generator=g) * 0.6, "k.conv": torch.randn(G * d, taps, generator=g) * 0.6, "v.conv": torch.randn(H * dv, taps, generator=g) * 0.6,
+            "A_log": torch.rand(H, generator=g) * 3.0 - 2.5 if a_log is None else torch.full((H,), a_log), "dt_bias": torch.randn(H, generator=g),
+            "norm": torch.rand(dv, generator=g) + 0.5}
+
+
+@pytest.mark.parametrize("H,G,d,dv,taps", [(3, 3, 40, 24, 4), (4, 2, 16, 64, 3), (1, 1, 130, 8, 1), (6, 2, 8, 33, 5), (2, 1, 64, 20, 2)])
+@pytest.mark.parametrize("cut_sizes", [[200], [1], [2, 5, 1, 3, 90], [7, 2]])
+def test_gated_delta_rule_under_cuts(dev, H, G, d, dv, taps, cut_sizes):
+    g = torch.Generator().manual_seed(H * d + taps)
+    m = {"heads": H, "kv_heads": G, "dim": d, "vdim": dv, "conv": taps}
+    w = _delta_weights(m, g)
+    lens = {2: 120, 0: 31, 1: 4}
+    N1 = 2 * G * d + 2 * H * dv + 2 * H
+    h = {s: torch.randn(T, N1, generator=g) for s, T in lens.items()}
+    got = _delta_run(dev, m, w, h, lens, cut_sizes, 1e-5)
+    for s in lens:
+        assert close(got[s], _delta_oracle(m, w, h[s], 1e-5), 5e-5), s
+
+
+@pytest.mark.parametrize("cut_sizes", [[500], [1], [64, 3]])
+def test_gated_delta_rule_keeps_its_first_write_over_hundreds_of_tokens(dev, cut_sizes):
+    """Decays next to one and later keys orthogonal to the first: what the first token wrote is still there 500 tokens later, when the
+    last query asks for it (a state lost at a cut, or a slot's stale state taken over, would show)."""
+    g = torch.Generator().manual_seed(7)
+    m = {"heads": 2, "kv_heads": 1, "dim": 12, "vdim": 10, "conv": 1}
+    w = _delta_weights(m, g, a_log=-9.0)
+    w["q.conv"], w["k.conv"], w["v.conv"] = torch.ones(12, 1), torch.ones(12, 1), torch.ones(20, 1)
+    T, N1 = 500, 2 * 12 + 2 * 20 + 4
+    h = torch.randn(T, N1, generator=g)
+    h[:, 12] = 0.0                                      # (silu(0) = 0: no later key has a part along the first one)
+    h[0, 12:24] = 0.0
+    h[0, 12] = 5.0
+    h[T - 1, 0] = 9.0                                   # the last query asks along the first key
+    h[:, 44:46] = 3.0                                   # strong writes
+    want = _delta_oracle(m, w, h, 1e-6)
+    forgot = _delta_oracle(m, w, h[1:], 1e-6)
+    assert float((want[-1] - forgot[-1]).abs().max()) > 0.2 * float(want[-1].abs().max())      # (the premise)
+    got = _delta_run(dev, m, w, {1: h}, {1: T}, cut_sizes, 1e-6)[1]
+    assert close(got, want, 1e-4)
+
+
+# =================================================== whole models =================================================================
+@pytest.mark.parametrize("name", list(SHAPES))
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_whole_prompt_and_residual_after_every_layer(dev, name, dtype):
+    whole_prompt(make_model(name, dtype, dev), name, tokens(name, 140, 1), dtype, slot=2, layers_too=True)
+
+
+@pytest.mark.parametrize("name", list(SHAPES))
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_cuts_batches_and_reuse(dev, name, dtype):
+    """Token by token from the first token; portions of changing size down to two tokens; four live requests of unequal length in a
+    pool that only fits with page reuse, more requests than slots over the run; a request left out of steps.  Every request's whole
+    prompt is checked against the oracle first; the schedules must then give the same logits."""
+    from vllm_i64_amd.engine import Engine
+    model = make_model(name, dtype, dev, max_tokens=4 * 64, max_seqs=4)
+    reqs = {"a": tokens(name, 61, 2), "b": tokens(name, 38, 3), "c": tokens(name, 1, 4), "d": tokens(name, 50, 5), "e": tokens(name, 33, 6), "f": tokens(name, 64, 7)}
+    want = {i: whole_prompt(model, name, t, dtype, slot=3) for i, t in reqs.items()}
+    eng = Engine(model)
+    got = replay(eng, {"b": reqs["b"]}, [[("b", 1)] for _ in range(38)])
+    assert same_to_rounding(got["b"], want["b"], dtype)
+    got = replay(eng, {"a": reqs["a"]}, [[("a", c)] for _, c in cuts_of(61, [2, 17, 1, 3, 16, 2, 5])])
+    assert same_to_rounding(got["a"], want["a"], dtype)
+    sched = [[("a", 30), ("b", 2)], [("a", 1), ("b", 20), ("c", 1), ("d", 7)], [("b", 1), ("d", 2), ("e", 16)], [("a", 28), ("b", 1), ("d", 1), ("e", 1)],
+             [("a", 2), ("b", 14), ("d", 40), ("e", 2)], [("e", 14), ("f", 33)], [("f", 1)], [("f", 30)]]
+    got = replay(eng, reqs, sched)
+    for i in reqs:
+        assert same_to_rounding(got[i], want[i], dtype), i
+    assert model.kv.free_blocks == model.kv.num_blocks and not eng.seqs
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_prefill_equals_token_by_token_to_rounding(dev, dtype):
+    from vllm_i64_amd.engine import Engine
+    name = "wide"
+    toks = tokens(name, 90, 12)
+    eng = Engine(make_model(name, dtype, dev, max_tokens=3 * 96, max_seqs=3))
+    whole = replay(eng, {"x": toks}, [[("x", 90)]])["x"]
+    single = replay(eng, {"y": toks}, [[("y", 1)] for _ in range(90)])["y"]
+    parts = replay(eng, {"z": toks}, [[("z", c)] for _, c in cuts_of(90, [2, 31, 1, 16])])["z"]
+    assert same_to_rounding(single, whole, dtype) and same_to_rounding(parts, whole, dtype)
+
+
+@pytest.mark.parametrize("name", ["odd", "wide"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_past_many_pages(dev, name, dtype):
+    from vllm_i64_amd.engine import Engine
+    toks = tokens(name, 300, 8)
+    model = make_model(name, dtype, dev, max_tokens=304, max_seqs=1)
+    want = whole_prompt(model, name, toks, dtype)
+    got = replay(Engine(model), {"x": toks}, [[("x", 9)]] + [[("x", 1)] for _ in range(291)])
+    assert same_to_rounding(got["x"], want, dtype)
+
+
+@pytest.mark.parametrize("name", ["odd", "plain", "twotap"])
+def test_greedy_generation_through_the_engine(dev, name):
+    """More prompts than slots; the engine's own scheduler, batching and sampling; against the oracle's greedy continuation."""
+    from vllm_i64_amd.engine import Engine, SamplingParams
+    model = make_model(name, "float32", dev, max_tokens=3 * 64, max_seqs=2)
+    prompts = [tokens(name, n, 20 + n) for n in (5, 19, 1, 12)]
+    new = 6
+    want = []
+    for p in prompts:
+        t = list(p)
+        for _ in range(new):
+            t.append(int(oracle_logits(name, t)[-1].argmax()))
+        want.append(t[len(p):])
+    eng = Engine(model, max_batch_tokens=16)
+    assert eng.generate(prompts, SamplingParams(max_new_tokens=new)) == want
+
+
+def test_graph_decoder_steps_match_the_oracle(dev):
+    """The batch decoder (a captured HIP graph replayed per step) from the first token on: previous tokens, shifted rows, convolution
+    inputs, the delta rule's state and the pages advance inside the graph."""
+    from vllm_i64_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("the batch decoder takes its argmax from the first library, which is not built")
+    from vllm_i64_amd.model import GreedyDecoder
+    name = "odd"
+    model = make_model(name, "float32", dev, max_tokens=256, max_seqs=3)
+    prompts = [tokens(name, n, 40 + n) for n in (4, 11, 7)]
+    dec = GreedyDecoder(model, 3, use_graph=True)
+    dec.prefill([torch.tensor(p) for p in prompts], reserve_extra=8)
+    seqs = [list(p) + [int(t)] for p, t in zip(prompts, dec.tokens.tolist())]
+    for _ in range(5):
+        dec.step()
+        torch.cuda.synchronize()
+        for s, t in zip(seqs, dec.tokens.tolist()):
+            s.append(int(t))
+    for p, s in zip(prompts, seqs):
+        t = list(p)
+        for _ in range(6):
+            t.append(int(oracle_logits(name, t)[-1].argmax()))
+        assert s == t
+
+
+def test_trace_command_on_a_checkpoint_folder(dev, tmp_path):
+    from safetensors.torch import save_file
+    name = "twotap"
+    ck = tmp_path / "ck"
+    ck.mkdir()
+    (ck / "config.json").write_text(json.dumps(config_of(name)))
+    save_file(make_weights(name), str(ck / "model.safetensors"))
+    toks = tokens(name, 21, 9)
+    steps = [{"step": 0, "entries": [{"id": "q", "tokens": toks[:10], "want": [0, 9]}], "end": []},
+             {"step": 1, "entries": [{"id": "q", "tokens": toks[10:12], "want": []}], "end": []},
+             {"step": 2, "entries": [{"id": "q", "tokens": toks[12:], "want": [8]}, {"id": "r", "tokens": toks[:3], "want": [2]}], "end": ["q", "r"]}]
+    out = tmp_path / "out"
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", str(ck), "--dtype", "float32", "--out", str(out), "--max-tokens", "128"],
+                       input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [l for l in r.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2"]
+    import numpy as np
+    want = oracle_logits(name, toks)
+    V = SHAPES[name]["vocab"]
+    a = torch.from_numpy(np.fromfile(out / "0.f32", dtype="<f4").reshape(-1, V))
+    c = torch.from_numpy(np.fromfile(out / "2.f32", dtype="<f4").reshape(-1, V))
+    assert not (out / "1.f32").exists()
+    assert agrees(a, want[[0, 9]], "float32") and agrees(c, torch.stack([want[20], want[2]]), "float32")

@@ -1,7 +1,8 @@
-"""`bench.py --design morilorn | dogalorn | zabutar`: prefill and decode throughput of a registered design at layer sizes of real models
+"""`bench.py --design morilorn | dogalorn | zabutar | fukatar`: prefill and decode throughput of a registered design at layer sizes of real models
 (random weights), beside the package's closest existing model at equal width, depth, feed-forward size and batch (Morilorn: the dense
 int8 decoder; Dogalorn: Morilorn, which shares its library, bf16 Linears and 32-bit residual; Zabutar: Dogalorn, the other design of
-recurrent layers beside attention with a distance bias), and the design's kernels one by one against their rooflines beside the like
+recurrent layers beside attention with a distance bias; Fukatar: Zabutar, the other design with a norm behind every sublayer, a matrix-valued
+recurrence and attention over separate keys and values), and the design's kernels one by one against their rooflines beside the like
 kernel of that model.  Prints one JSON line."""
 from __future__ import annotations
 
@@ -524,6 +525,187 @@ def run_zabutar(args) -> dict:
     return result
 
 
+FUKATAR_SIZES = {
+    "w1024": dict(width=1024, blocks=4, heads=16, kv_heads=4, dim=64, vdim=64, rot_dims=64, lat_heads=16, lat_dim=64, lat_vdim=64, kv_rank=256, rec_heads=8,
+                  rec_kv_heads=4, rec_dim=128, rec_vdim=128, taps=4, ff=4096),
+    "w2048": dict(width=2048, blocks=2, heads=32, kv_heads=8, dim=64, vdim=64, rot_dims=64, lat_heads=32, lat_dim=64, lat_vdim=64, kv_rank=256, rec_heads=16,
+                  rec_kv_heads=8, rec_dim=128, rec_vdim=128, taps=4, ff=8192),
+}
+
+
+def _fukatar_kernels(sz, rows, batch, ctx, dev):
+    """Single launches at the step's shapes with the share of their roofline (matrix products: bf16 matrix peak; recurrences: the larger of
+    bytes / HBM rate and flop / fp32 vector rate; everything else: bytes / HBM rate), each beside the like kernel of Zabutar (of Morilorn
+    for the latent attention, of Dogalorn for the convolution with silu)."""
+    from . import ops_dense as D
+    W, ff, H, G, dm, dv = sz["width"], sz["ff"], sz["heads"], sz["kv_heads"], sz["dim"], sz["vdim"]
+    Hr, Gr, dk, dr, taps = sz["rec_heads"], sz["rec_kv_heads"], sz["rec_dim"], sz["rec_vdim"], sz["taps"]
+    Hl, dl, r = sz["lat_heads"], sz["lat_dim"], sz["kv_rank"]
+    out = {}
+    g = torch.Generator(device=dev).manual_seed(1)
+    rn = lambda *s: torch.randn(*s, device=dev, generator=g)
+
+    def row(name, t, flops=0.0, bytes_=0.0, peak=BF16_TFLOPS):
+        share = max(flops / t / (peak * 1e12), bytes_ / t / (HBM_GBS * 1e9))
+        out[name] = {"us": round(t * 1e6, 1), "roofline_share": round(share, 3)}
+
+    seq = 512
+    warm_a, warm_w, warm_c = rn(rows, W), (rn(W, W) * 0.02).to(torch.bfloat16), torch.empty(rows, W, device=dev)
+    _time(lambda: D.linear(warm_a, warm_w, warm_c), 20)      # clocks and caches settle before the first timed launch
+    for n, tag in ((rows, "prefill"), (batch, "decode")):
+        nseq = n // seq if tag == "prefill" else n
+        per = seq if tag == "prefill" else 1
+        pos0 = 0 if tag == "prefill" else ctx - 1
+        pos = (torch.arange(per, dtype=torch.int32) + pos0).repeat(nseq).to(dev)
+        slots = torch.arange(nseq, dtype=torch.int32).repeat_interleave(per).to(dev)
+        seg = (torch.arange(nseq + 1, dtype=torch.int32) * per).to(dev)
+        single = tag == "decode"
+        reps = 5 if tag == "prefill" else 20
+        a = rn(n, W)
+        # feed-forward: up-projection with the squared relu; beside the same Linear with Zabutar's bias and two-branch activation
+        w_up, b_up = (rn(ff, W) * 0.02).to(torch.bfloat16), rn(ff)
+        act = torch.empty(n, ff, device=dev)
+        t = _time(lambda: D.linear(a, w_up, act, epilogue=D.EPI_RELU_SQ), reps)
+        row(f"linear_up_relu_sq_{tag}", t, flops=2.0 * n * ff * W, bytes_=2.0 * ff * W + 4.0 * n * (W + ff))
+        t = _time(lambda: D.linear(a, w_up, act, bias=b_up, epilogue=D.EPI_XIELU, act_a=0.7, act_b=1.2), reps)
+        row(f"zabutar_linear_up_bias_xielu_{tag}", t, flops=2.0 * n * ff * W, bytes_=2.0 * ff * W + 4.0 * n * (W + ff))
+        # residual: the centred norm of one result, and of the mean of two normed results, added; beside Zabutar's norm behind + norm in front
+        st, y, y2, h = rn(1, n, W), rn(n, W), rn(n, W), torch.empty(n, W, device=dev)
+        wn, one = torch.ones(W, device=dev), torch.ones(1, device=dev)
+        t = _time(lambda: D.streams_step(st, y=y, y_eps=1e-6, out_w=one, post_w=wn, post_center=True), reps)
+        row(f"residual_centred_norm_{tag}", t, bytes_=4.0 * n * W * 3)
+        t = _time(lambda: D.streams_step(st, y=y, y2=y2, yn_w=wn, y2n_w=wn, y_eps=1e-6, out_w=one, post_w=wn, post_center=True), reps)
+        row(f"residual_two_results_centred_norm_{tag}", t, bytes_=4.0 * n * W * 4)
+        t = _time(lambda: D.streams_step(st, y=y, yn_w=wn, y_eps=1e-6, out_w=one, norm_w=wn, eps=1e-6, h=h), reps)
+        row(f"zabutar_sandwich_residual_{tag}", t, bytes_=4.0 * n * W * 4)
+        # token shift (two taps added to the input); beside Zabutar's four-tap added convolution
+        sw, sstate, hs = rn(W, 2) * 0.5, torch.zeros(nseq, 1, W, device=dev), torch.empty(n, W, device=dev)
+        t = _time(lambda: D.causal_conv(a, off=0, channels=W, w=sw, bias=None, positions=pos, slot_ids=slots, state=sstate, out=hs, n=n, added=True, single_rows=single), reps)
+        row(f"token_shift_{tag}", t, bytes_=4.0 * n * W * 2)
+        cw, cstate = rn(W, 4) * 0.1, torch.zeros(nseq, 3, W, device=dev)
+        t = _time(lambda: D.causal_conv(a, off=0, channels=W, w=cw, bias=None, positions=pos, slot_ids=slots, state=cstate, out=hs, n=n, added=True, single_rows=single), reps)
+        row(f"zabutar_input_conv_{tag}", t, bytes_=4.0 * n * W * 2)
+        # rotated attention: prep (norms, rotation of q, k and v, cache write), attention with capped scores, the turn back + gate
+        plen = seq if tag == "prefill" else ctx
+        nb = (plen + 15) // 16
+        bt = torch.arange(nseq * nb, dtype=torch.int32, device=dev).view(nseq, nb).contiguous()
+        gs = dv + dm
+        kc = (rn(nseq * nb, 16, G * gs) * 0.5).to(torch.bfloat16)
+        nq, nk, nv = H * dm, G * dm, G * dv
+        ldp = nq + nk + nv + H
+        P = rn(n, ldp) * 0.3
+        q, oa = torch.empty(n, H * gs, device=dev), torch.empty(n, H * dv, device=dev)
+        inv = torch.rand(dm // 2, device=dev, generator=g)
+        vfr = torch.rand(dv // 2, device=dev, generator=g)
+        qw, kw = torch.ones(nq, device=dev), torch.ones(nk, device=dev)
+        t = _time(lambda: D.rot_prep(P, q_off=0, k_off=nq, v_off=nq + nk, heads=H, kv_heads=G, dim=dm, vdim=dv, q_norm_w=qw, k_norm_w=kw, eps=1e-6, rot_dims=dm,
+                                     interleaved=False, inv_freq=inv, rot_mult=1.1, head_norm=False, v_freq=vfr, scale=0.125, positions=pos, slot_ids=slots,
+                                     block_table=bt, cache=kc, q=q, n=n), reps)
+        row(f"rot_prep_{tag}", t, bytes_=4.0 * n * (nq + nk + nv + H * gs) + 2.0 * n * G * gs)
+        t = _time(lambda: D.kv_prep(P, q_off=0, k_off=nq, v_off=nq + nk, heads=H, kv_heads=G, dim=dm, vdim=dv, scale=0.125, positions=pos, slot_ids=slots, block_table=bt,
+                                    cache=kc, q=q, n=n), reps)
+        row(f"zabutar_kv_prep_{tag}", t, bytes_=4.0 * n * (nq + nk + nv + H * gs) + 2.0 * n * G * gs)
+        keys = seq * (seq + 1) / 2 * nseq if tag == "prefill" else float(ctx) * n
+        waves = 3072 if gs <= 64 else (2048 if gs <= 128 else 1024)
+        sp = 1 if tag == "prefill" else max(1, min(waves // max(1, n * G * ((H // G + 15) // 16)), int(keys / n) // 64, 64))
+        mode = 3 if tag == "prefill" else 2
+        t = _time(lambda: D.kattn(q, kc, None, bt, slots, pos, chunk=0, bias=None, sink=False, heads=H, kv_heads=G, dim=dm, vdim=dv, out=oa, n=n, mode=mode, splits=sp,
+                                  softcap=50.0), reps)
+        abytes = (2.0 * keys * G * gs if tag == "decode" else 0.0) + 4.0 * n * H * (gs + dv)
+        row(f"capped_attention_{tag}", t, flops=2.0 * keys * H * (dm + dv), bytes_=abytes)
+        bias = torch.zeros(4097, H, device=dev)
+        t = _time(lambda: D.kattn(q, kc, None, bt, slots, pos, chunk=0, bias=bias, sink=False, heads=H, kv_heads=G, dim=dm, vdim=dv, out=oa, n=n, mode=mode, splits=sp), reps)
+        row(f"zabutar_kv_attention_{tag}", t, flops=2.0 * keys * H * (dm + dv), bytes_=abytes)
+        t = _time(lambda: D.rot_post(oa, heads=H, vdim=dv, interleaved=False, v_freq=vfr, positions=pos, gate=P, gate_off=nq + nk + nv, ldg=ldp, n=n), reps)
+        row(f"rot_post_{tag}", t, bytes_=4.0 * n * H * dv * 2)
+        # latent attention with learned sinks; beside the same launch without them (Morilorn's)
+        lc = (rn(nseq * nb, 16, r) * 0.5).to(torch.bfloat16)
+        ql, ol = rn(n, Hl * r) * 0.1, torch.empty(n, Hl * r, device=dev)
+        sink = torch.zeros(Hl, device=dev)
+        spl = 1 if tag == "prefill" else max(1, min(1024 // max(1, n * ((Hl + 15) // 16)), int(keys / n) // 64, 64))
+        lflops, lbytes = 4.0 * keys * Hl * r, (2.0 * keys * r if tag == "decode" else 0.0) + 8.0 * n * Hl * r
+        t = _time(lambda: D.latent_attn(ql, lc, bt, slots, pos, window=0, scale=0.125, heads=Hl, kv_rank=r, rot_dim=0, out=ol, n=n, mode=mode, splits=spl, sink=sink), reps)
+        row(f"latent_attention_sink_{tag}", t, flops=lflops, bytes_=lbytes)
+        t = _time(lambda: D.latent_attn(ql, lc, bt, slots, pos, window=0, scale=0.125, heads=Hl, kv_rank=r, rot_dim=0, out=ol, n=n, mode=mode, splits=spl), reps)
+        row(f"morilorn_latent_attention_{tag}", t, flops=lflops, bytes_=lbytes)
+        # gated delta rule: convolution + silu, gates, scan, gated head norm; beside Dogalorn's convolution and Zabutar's gates, scan, head norm
+        rk, rv = Gr * dk, Hr * dr
+        C = 2 * rk + rv
+        Pr = rn(n, C + 2 * Hr + rv) * 0.5
+        cw2, cst2, X = rn(C, taps) * 0.3, torch.zeros(nseq, taps - 1, C, device=dev), torch.empty(n, C, device=dev)
+        t = _time(lambda: D.causal_conv(Pr, off=0, channels=C, w=cw2, bias=None, positions=pos, slot_ids=slots, state=cst2, out=X, n=n, single_rows=single), reps)
+        row(f"delta_conv_silu_{tag}", t, bytes_=4.0 * n * C * 2)
+        Gt = torch.empty(n, 2 * Hr, device=dev)
+        cols = dict(q_off=0, k_off=rk, v_off=2 * rk, heads=Hr, kv_heads=Gr, dim=dk, vdim=dr, n=n)
+        al, db = torch.linspace(-4.0, 0.0, Hr, device=dev), torch.zeros(Hr, device=dev)
+        t = _time(lambda: D.gdn_gates(X, Gt, Pr, b_off=C, a_off=C + Hr, a_log=al, dt_bias=db, unit_eps=1e-6, q_scale=dk ** -0.5, **cols), reps)
+        row(f"delta_gates_{tag}", t, bytes_=4.0 * n * rk * 4)
+        nkz = Hr * dk
+        Pz = rn(n, 2 * nkz + rv) * 0.5
+        lower = torch.rand(nkz, device=dev, generator=g) * 0.9
+        zc = dict(q_off=0, f_off=nkz, v_off=2 * nkz, heads=Hr, dim=dk, vdim=dr, n=n)
+        t = _time(lambda: D.gla_gates(Pz, lower=lower, q_act=True, **zc), reps)
+        row(f"zabutar_gla_gates_{tag}", t, bytes_=4.0 * n * nkz * 4)
+        dstate, ro, rg = torch.zeros(nseq, Hr, dr, dk, device=dev), torch.empty(n, rv, device=dev), torch.empty(n, rv, device=dev)
+        t = _time(lambda: D.gdn_scan(X, Gt, seg_start=seg, nseg=nseq, positions=pos, slot_ids=slots, state=dstate, out=ro, **cols), reps)
+        row(f"delta_scan_{tag}", t, flops=7.0 * n * Hr * dk * dr, bytes_=4.0 * n * (2 * rk + 2 * rv) + 8.0 * nseq * Hr * dk * dr, peak=F32_TFLOPS)
+        Pz.uniform_(0.0, 1.0)
+        t = _time(lambda: D.gla_scan(Pz, seg_start=seg, nseg=nseq, positions=pos, slot_ids=slots, state=dstate, out=ro, **zc), reps)
+        row(f"zabutar_gla_scan_{tag}", t, flops=5.0 * n * Hr * dk * dr, bytes_=4.0 * n * (2 * nkz + 2 * rv) + 8.0 * nseq * Hr * dk * dr, peak=F32_TFLOPS)
+        nwv = torch.ones(dr, device=dev)
+        t = _time(lambda: D.gate_norm(ro, nwv, rg, groups=Hr, eps=1e-6, z=Pr, z_off=C + 2 * Hr, ldz=C + 2 * Hr + rv, n=n, gate_after=True, width=rv), reps)
+        row(f"gated_head_norm_{tag}", t, bytes_=4.0 * n * rv * 3)
+        t = _time(lambda: D.gate_norm(ro, torch.ones(rv, device=dev), rg, groups=Hr, eps=1e-6, n=n), reps)
+        row(f"zabutar_head_norm_{tag}", t, bytes_=4.0 * n * rv * 2)
+    return out
+
+
+def run_fukatar(args) -> dict:
+    from . import _lib, synth
+    from .fukatar import FukatarModel
+    from .model import GreedyDecoder
+    from .zabutar import ZabutarModel
+    _lib.load(), _lib.load_dense()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    batch, ctx, rows = args.batch, args.prompt_len, 4096
+    result = {"metric": "prefill / decode tokens/s of the Fukatar design beside Zabutar at equal sizes", "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+              "warmup": args.warmup, "dtype": "bf16 matrix products, fp32 residual / norms / recurrences / attention math (both designs)", "data": "synthetic",
+              "config": {"batch": batch, "context": ctx, "prefill_step": f"{rows} rows = {rows // 512} prompts of 512 tokens"}, "sizes": {}}
+    for name in (args.design_sizes.split(",") if args.design_sizes else sorted(FUKATAR_SIZES)):
+        sz = FUKATAR_SIZES[name]
+        need_tokens = batch * (ctx + args.steps + args.warmup + 64)
+
+        def fill(m):
+            g = torch.Generator(device=dev).manual_seed(5)
+            for t in {id(t): t for t in m.kv.rows if t is not None}.values():
+                t.copy_((0.5 * torch.randn(t.shape, device=dev, generator=g)).to(t.dtype))
+            for d in m.kv.state:
+                for t in d.values():
+                    t.copy_(0.1 * torch.randn(t.shape, device=dev, generator=g))
+
+        cfg = synth.fukatar_config(**sz)
+        model = FukatarModel(cfg, synth.make_fukatar_weights(cfg), device=dev, dtype="bfloat16", max_seqs=batch, num_kv_blocks=need_tokens // 16)
+        p, d, ms = _steps(model, GreedyDecoder, batch, ctx, rows, 512, args.steps, args.warmup, fill, cfg.vocab, dev)
+        entry = {"fukatar": {"prefill_tokens_per_s": round(p, 1), "decode_tokens_per_s": round(d, 1), "decode_ms_per_step": round(ms, 3), "layers": cfg.num_layers,
+                             "shape": sz}}
+        del model
+        torch.cuda.empty_cache()
+        zs = ZABUTAR_SIZES[name]
+        zcfg = synth.zabutar_config(max_positions=max(4096, ctx + args.steps + args.warmup + 64), **zs)
+        zm = ZabutarModel(zcfg, synth.make_zabutar_weights(zcfg), device=dev, dtype="bfloat16", max_seqs=batch, num_kv_blocks=need_tokens // 16)
+        p, d, ms = _steps(zm, GreedyDecoder, batch, ctx, rows, 512, args.steps, args.warmup, fill, zcfg.vocab, dev)
+        entry["zabutar"] = {"prefill_tokens_per_s": round(p, 1), "decode_tokens_per_s": round(d, 1), "decode_ms_per_step": round(ms, 3), "layers": zcfg.num_layers}
+        del zm
+        torch.cuda.empty_cache()
+        entry["kernels"] = _fukatar_kernels(sz, rows, batch, ctx, dev)
+        result["sizes"][name] = entry
+    first = result["sizes"][sorted(result["sizes"])[0]]["fukatar"]
+    result["value"], result["ms_per_step"] = first["decode_tokens_per_s"], first["decode_ms_per_step"]
+    result["higher_is_better"], result["scaling"], result["vs_baseline"] = True, "weak", None
+    return result
+
+
 def main(args) -> int:
-    print(json.dumps({"dogalorn": run_dogalorn, "zabutar": run_zabutar}.get(args.design, run)(args)), flush=True)
+    print(json.dumps({"dogalorn": run_dogalorn, "zabutar": run_zabutar, "fukatar": run_fukatar}.get(args.design, run)(args)), flush=True)
     return 0

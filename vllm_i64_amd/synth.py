@@ -218,3 +218,61 @@ def make_zabutar_weights(cfg, seed: int = 0, std: float = 0.02) -> Dict[str, tor
             if f.shared_ff:
                 w.update({p + "mlp.shared.gate": rn(f.shared_ff, W), p + "mlp.shared.up": rn(f.shared_ff, W), p + "mlp.shared.down": rn(W, f.shared_ff)})
     return w
+
+
+def fukatar_config(width: int = 1024, blocks: int = 4, heads: int = 16, kv_heads: int = 4, dim: int = 64, vdim: int = 64, rot_dims: int = 64, lat_heads: int = 16,
+                   lat_dim: int = 64, lat_vdim: int = 64, kv_rank: int = 256, rec_heads: int = 8, rec_kv_heads: int = 4, rec_dim: int = 128, rec_vdim: int = 128,
+                   taps: int = 4, ff: int = 4096, vocab: int = 32000):
+    """A Fukatar configuration with layers of a real model's proportions: `blocks` times (rotated attention with gated heads, latent
+    attention, attention beside a gated delta rule, latent attention), every layer with a dense feed-forward; random weights:
+    make_fukatar_weights."""
+    from .config import FukatarConfig
+    mlp = {"kind": "dense", "ff": ff}
+    att = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5, "softcap": 50.0,
+           "rot": {"base": 10000.0, "dims": rot_dims, "scaling": {"factor": 8.0, "original": 2048, "fast": 32.0, "slow": 1.0}}}
+    left = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5, "softcap": 30.0, "rot": {"base": 10000.0, "dims": rot_dims // 2}}
+    right = {"heads": rec_heads, "kv_heads": rec_kv_heads, "dim": rec_dim, "vdim": rec_vdim, "conv": taps}
+    lat = {"heads": lat_heads, "dim": lat_dim, "vdim": lat_vdim, "kv_rank": kv_rank, "scale": lat_dim ** -0.5}
+    layers = []
+    for _ in range(blocks):
+        layers += [{"type": "attention", "mixer": att, "mlp": mlp}, {"type": "latent_attention", "mixer": lat, "mlp": mlp},
+                   {"type": "parallel", "mixer": {"left": left, "right": right}, "mlp": mlp}, {"type": "latent_attention", "mixer": lat, "mlp": mlp}]
+    return FukatarConfig.from_dict({"architecture": "Fukatar", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
+                                    "embedding": {"scale": width ** 0.5, "bigram": {"buckets": 8191, "mul_prev": 1000003, "mul_cur": 31}}, "layers": layers})
+
+
+def make_fukatar_weights(cfg, seed: int = 0, std: float = 0.02) -> Dict[str, torch.Tensor]:
+    """bf16 N(0, std) matrices, norm weights one, shifts one half, convolution taps small, sinks zero, decays spread over the heads."""
+    g = torch.Generator().manual_seed(seed)
+    W = cfg.width
+
+    def rn(*shape, s=std):
+        return torch.empty(*shape, dtype=torch.float32).normal_(0.0, s, generator=g).to(torch.bfloat16)
+
+    one = lambda *n: torch.ones(*n, dtype=torch.bfloat16)
+    w = {"embed": rn(cfg.vocab, W), "head": rn(cfg.vocab, W), "final.norm": one(W)}
+    if cfg.bigram is not None:
+        w["bigram"] = rn(cfg.bigram.buckets + 1, W)
+    for i, L in enumerate(cfg.layers):
+        p, m = f"l{i}.", L.mixer
+        w.update({p + "norm1": one(W), p + "shift": one(W) * 0.5})
+        if L.mlp is not None:
+            w.update({p + "norm2": one(W), p + "mlp.up": rn(L.mlp.ff, W), p + "mlp.down": rn(W, L.mlp.ff)})
+        if L.type == "latent_attention":
+            H, r = m.heads, m.kv_rank
+            w.update({p + "mix.q": rn(H * m.dim, W), p + "mix.dkv": rn(r, W), p + "mix.dkv.norm": one(r), p + "mix.uk": rn(H * m.dim, r), p + "mix.uv": rn(H * m.vdim, r),
+                      p + "mix.sink": torch.zeros(H, dtype=torch.bfloat16), p + "mix.o": rn(W, H * m.vdim)})
+            continue
+        a, ap = (m, p + "mix.") if L.type == "attention" else (m.left, p + "mix.left.")
+        nq, nk, nv = a.heads * a.dim, a.kv_heads * a.dim, a.kv_heads * a.vdim
+        w.update({ap + "q": rn(nq, W), ap + "k": rn(nk, W), ap + "v": rn(nv, W), ap + "o": rn(W, a.heads * a.vdim)})
+        if L.type == "attention":
+            w.update({ap + "q.norm": one(nq), ap + "k.norm": one(nk), ap + "g": rn(a.heads, W)})
+        else:
+            r, rp = m.right, p + "mix.right."
+            rk, rv = r.kv_heads * r.dim, r.heads * r.vdim
+            w.update({rp + "q": rn(rk, W), rp + "k": rn(rk, W), rp + "v": rn(rv, W), rp + "q.conv": rn(rk, r.conv, s=0.3), rp + "k.conv": rn(rk, r.conv, s=0.3),
+                      rp + "v.conv": rn(rv, r.conv, s=0.3), rp + "b": rn(r.heads, W), rp + "a": rn(r.heads, W),
+                      rp + "A_log": torch.linspace(-4.0, 0.0, r.heads).to(torch.bfloat16), rp + "dt_bias": torch.zeros(r.heads, dtype=torch.bfloat16),
+                      rp + "norm": one(r.vdim), rp + "g": rn(rv, W), rp + "o": rn(W, rv), p + "mix.left.out": one(W), p + "mix.right.out": one(W)})
+    return w
