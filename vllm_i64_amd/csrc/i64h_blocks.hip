@@ -545,7 +545,8 @@ int i64h_gdn_scan(const i64h_gdn_args* dp, void* stream) {
     if (d.nseg <= 0 || d.n == 0) return 0;
     const int kpt = (d.dim + 15) / 16;
     // columns per lane: query and key are loaded once for both - unless the launch would then leave most of the chip idle
-    const int cpt = (d.vdim > 16 && (int64_t)d.heads * ((d.vdim + 31) / 32) * d.nseg >= 512) ? 2 : 1;
+    // (two columns also give the two row sums of a token independent work to overlap: measured faster from 256 workgroups on)
+    const int cpt = (d.vdim > 16 && (int64_t)d.heads * ((d.vdim + 31) / 32) * d.nseg >= 256) ? 2 : 1;
     const int ctiles = (d.vdim + 16 * cpt - 1) / (16 * cpt);
     const dim3 grid((unsigned)(d.heads * ctiles), (unsigned)d.nseg);
     auto launch = [&](auto kern, int K) {

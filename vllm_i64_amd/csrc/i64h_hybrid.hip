@@ -12,6 +12,8 @@
 //   kattn_row_kernel      : attention over the cached keys (which are also the values, or with the values in front of them in the
 //                           same cached row) with distance bias, chunk mask and sink
 //   kv_prep_kernel        : [q | k | v] projections -> the cached row [v | k] per key head and query rows with zeros in the value columns
+//   rot_prep_kernel       : the same with whole-row or per-head query / key norms, rotation of a part of every head in either pair layout
+//                           and values turned by their own position; rot_post_kernel turns a head's sum back and applies a gate per head
 // A row continues the row before it iff slot and position say so; state is taken as empty at position 0.  All arithmetic fp32.
 #include "i64h_common.h"
 #include "i64h_dense.h"
@@ -576,8 +578,8 @@ __global__ __launch_bounds__(256) void kv_prep_kernel(const i64h_kv_prep_args p)
 
 // ---------------------------------------------------------------------------------------------------------------------------
 // [q | k | v] projections -> whole-row norms, rotation (two pair layouts, a part of every head), per-head norms, rotated values ->
-// the paged cache row [v | k] per key head and the query rows [0 | q * scale].  One workgroup per token; the normed and rotated
-// queries and keys wait in LDS for the per-head sums.
+// the paged cache row [v | k] per key head and the query rows [0 | q * scale].  The normed and rotated queries and keys wait in LDS
+// for the per-head sums.
 __device__ __forceinline__ void rot_pair(int d, int dims, int interleaved, int& a, int& b, int& i, bool& second) {
     // the pair of dimension d < dims: a the first member, b the second, i the pair's index; second: d is b
     if (interleaved) {
@@ -588,112 +590,132 @@ __device__ __forceinline__ void rot_pair(int d, int dims, int interleaved, int& 
     }
 }
 
+// One workgroup per token, two passes: the raw queries and keys go to LDS while their squares are summed (a rotation keeps the sum of
+// squares of a pair, so the per-head sums behind the rotation are those in front of it, the rotated part times rot_mult^2); the second
+// pass norms and rotates out of LDS straight into the query rows and the cached row.
 __global__ __launch_bounds__(256) void rot_prep_kernel(const i64h_rot_prep_args p) {
-    extern __shared__ float sv[];   // [heads * dim] queries, [kv_heads * dim] keys, [heads + kv_heads] 1 / rms per head, 4 for reductions
+    extern __shared__ float sv[];   // [heads * dim + kv_heads * dim] raw queries and keys, [heads + kv_heads] 1 / rms per head, 8 for
+                                    // reductions, [rot_dims] cosines and sines of the row's angles, [vdim] those of the values' angles
     const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
     const int64_t t = blockIdx.x;
     const int dim = p.dim, vd = p.vdim, gs = vd + dim;
     const int nq = p.heads * dim, nk = p.kv_heads * dim;
+    const int half = p.rot_dims >> 1, vhalf = p.v_freq ? vd >> 1 : 0;
     float* inv = sv + nq + nk;
     float* red = inv + p.heads + p.kv_heads;
+    float* rcs = red + 8;           // [half] cosines, [half] sines: every head turns by the same angles
+    float* vcs = rcs + 2 * half;    // [vhalf] cosines, [vhalf] sines
     const float* q = p.P + t * p.ldp + p.q_off;
     const float* k = p.P + t * p.ldp + p.k_off;
     const float* v = p.P + t * p.ldp + p.v_off;
     const int pos = p.positions[t];
     const float fpos = (float)pos;
-    float qr = 1.0f, kr = 1.0f;
-    if (p.q_norm_w) {
-        float a = 0.0f, b = 0.0f;
-        for (int c = tid; c < nq; c += 256) a += q[c] * q[c];
-        for (int c = tid; c < nk; c += 256) b += k[c] * k[c];
-        a = hy_block_sum(a, red);
-        b = hy_block_sum(b, red);
-        qr = 1.0f / sqrtf(a / (float)nq + p.eps);
-        kr = 1.0f / sqrtf(b / (float)nk + p.eps);
-    }
+    float a = 0.0f, b = 0.0f;
     for (int c = tid; c < nq + nk; c += 256) {
-        const bool isq = c < nq;
-        const int e = isq ? c : c - nq;
-        const int h0 = (e / dim) * dim, d = e % dim;
-        const float* src = isq ? q : k;
-        const float* nw = isq ? p.q_norm_w : p.k_norm_w;
-        const float r = isq ? qr : kr;
-        auto val = [&](int idx) { return nw ? src[idx] * r * nw[idx] : src[idx]; };
-        float o;
-        if (d < p.rot_dims) {
-            int a, b, i;
-            bool second;
-            rot_pair(d, p.rot_dims, p.interleaved, a, b, i, second);
-            float sn, cs;
+        const float x = c < nq ? q[c] : k[c - nq];
+        sv[c] = x;
+        if (c < nq) a += x * x;
+        else b += x * x;
+    }
+    for (int i = tid; i < half + vhalf; i += 256) {
+        float sn, cs;
+        if (i < half) {
             sincosf(fpos * p.inv_freq[i], &sn, &cs);
-            sn *= p.rot_mult, cs *= p.rot_mult;
-            const float u = val(h0 + a), w = val(h0 + b);
-            o = second ? w * cs + u * sn : u * cs - w * sn;
+            rcs[i] = cs * p.rot_mult, rcs[half + i] = sn * p.rot_mult;
         } else {
-            o = val(h0 + d);
+            sincosf(fpos * p.v_freq[i - half], &sn, &cs);
+            vcs[i - half] = cs, vcs[vhalf + i - half] = sn;
         }
-        sv[c] = o;
+    }
+    float qr = 1.0f, kr = 1.0f;
+    if (p.q_norm_w) {   // (both sums through one exchange)
+        a = wave_sum(a), b = wave_sum(b);
+        __syncthreads();
+        if (lane == 0) red[wid] = a, red[4 + wid] = b;
+        __syncthreads();
+        qr = 1.0f / sqrtf((red[0] + red[1] + red[2] + red[3]) / (float)nq + p.eps);
+        kr = 1.0f / sqrtf((red[4] + red[5] + red[6] + red[7]) / (float)nk + p.eps);
     }
     __syncthreads();
     if (p.head_norm) {
+        const float m2 = p.rot_mult * p.rot_mult;
         for (int h = wid; h < p.heads + p.kv_heads; h += 4) {
             float s = 0.0f;
-            for (int d = lane; d < dim; d += 64) s += sv[h * dim + d] * sv[h * dim + d];
+            for (int d = lane; d < dim; d += 64) {
+                const float x = sv[h * dim + d];
+                s += d < p.rot_dims ? x * x * m2 : x * x;
+            }
             s = wave_sum(s);
             if (lane == 0) inv[h] = 1.0f / sqrtf(s / (float)dim + p.eps);
         }
         __syncthreads();
     }
     float* Q = p.Q + t * p.heads * gs;
-    for (int c = tid; c < p.heads * gs; c += 256) {
-        const int h = c / gs, d = c % gs;
-        float o = 0.0f;
-        if (d >= vd) {
-            o = sv[h * dim + d - vd];
-            if (p.head_norm) o *= inv[h];
-            o *= p.scale;
-        }
-        Q[c] = o;
-    }
     const int64_t cr = cache_row(p.block_table, p.max_blocks_per_seq, p.block_size, p.slot_ids[t], pos);
     const int nkv = p.kv_heads * gs;
-    for (int c = tid; c < nkv; c += 256) {
-        const int g = c / gs, d = c % gs;
+    // every head's part of a query row and of the cached row: [vdim zeros or values | dim rotated values]
+    for (int c = tid; c < (p.heads + p.kv_heads) * gs; c += 256) {
+        const int h = c / gs, d = c % gs;
+        const bool isq = h < p.heads;
         float o;
         if (d >= vd) {
-            o = sv[nq + g * dim + d - vd];
-            if (p.head_norm) o *= inv[p.heads + g];
-        } else if (p.v_freq) {
-            int a, b, i;
-            bool second;
-            rot_pair(d, vd, p.interleaved, a, b, i, second);
-            float sn, cs;
-            sincosf(fpos * p.v_freq[i], &sn, &cs);
-            const float u = v[g * vd + a], w = v[g * vd + b];
-            o = second ? w * cs + u * sn : u * cs - w * sn;
+            const int e = d - vd, h0 = h * dim;      // (the keys' raw values lie behind the queries': head index heads + g)
+            const float* nw = isq ? p.q_norm_w : p.k_norm_w;
+            const float r = isq ? qr : kr;
+            const int w0 = isq ? h0 : h0 - nq;
+            auto val = [&](int idx) { return nw ? sv[h0 + idx] * r * nw[w0 + idx] : sv[h0 + idx]; };
+            if (e < p.rot_dims) {
+                int ia, ib, i;
+                bool second;
+                rot_pair(e, p.rot_dims, p.interleaved, ia, ib, i, second);
+                const float cs = rcs[i], sn = rcs[half + i];
+                const float u = val(ia), w = val(ib);
+                o = second ? w * cs + u * sn : u * cs - w * sn;
+            } else {
+                o = val(e);
+            }
+            if (p.head_norm) o *= inv[h];
+            if (isq) o *= p.scale;
+        } else if (isq) {
+            o = 0.0f;
         } else {
-            o = v[g * vd + d];
+            const int g = h - p.heads;
+            if (p.v_freq) {
+                int ia, ib, i;
+                bool second;
+                rot_pair(d, vd, p.interleaved, ia, ib, i, second);
+                const float cs = vcs[i], sn = vcs[vhalf + i];
+                const float u = v[g * vd + ia], w = v[g * vd + ib];
+                o = second ? w * cs + u * sn : u * cs - w * sn;
+            } else {
+                o = v[g * vd + d];
+            }
         }
-        if (p.cache_dtype == 0) ((float*)p.cache)[cr * nkv + c] = o;
-        else ((__bf16*)p.cache)[cr * nkv + c] = (__bf16)o;
+        if (isq) Q[c] = o;
+        else if (p.cache_dtype == 0) ((float*)p.cache)[cr * nkv + c - p.heads * gs] = o;
+        else ((__bf16*)p.cache)[cr * nkv + c - p.heads * gs] = (__bf16)o;
     }
 }
 
 // the attention output of every head turned back by the row's own position and multiplied by the head's sigmoid gate, in place:
 // a thread takes whole pairs
 __global__ __launch_bounds__(256) void rot_post_kernel(const i64h_rot_post_args p) {
+    extern __shared__ float sv[];   // [vdim / 2] cosines, [vdim / 2] sines: every head turns by the same angles
     const int64_t t = blockIdx.x;
     const int vd = p.vdim, half = vd >> 1;
-    const float fpos = (float)p.positions[t];
     float* O = p.O + t * p.heads * vd;
+    if (p.v_freq) {
+        const float fpos = (float)p.positions[t];
+        for (int i = threadIdx.x; i < half; i += 256) sincosf(fpos * p.v_freq[i], &sv[half + i], &sv[i]);
+        __syncthreads();
+    }
     const int items = p.v_freq ? p.heads * half : p.heads * vd;
     for (int e = threadIdx.x; e < items; e += 256) {
         if (p.v_freq) {
             const int h = e / half, i = e % half;
             const int a = p.interleaved ? 2 * i : i, b = p.interleaved ? 2 * i + 1 : i + half;
             const float g = p.gate ? hy_sigmoid(p.gate[t * p.ldg + h]) : 1.0f;
-            float sn, cs;
-            sincosf(fpos * p.v_freq[i], &sn, &cs);
+            const float cs = sv[i], sn = sv[half + i];
             const float u = O[h * vd + a], w = O[h * vd + b];
             O[h * vd + a] = (u * cs + w * sn) * g;      // the turn by the negative angle
             O[h * vd + b] = (w * cs - u * sn) * g;
@@ -902,7 +924,7 @@ int i64h_rot_prep(const i64h_rot_prep_args* dp, void* stream) {
     I64H_CHECK_ARG((d.q_norm_w == nullptr) == (d.k_norm_w == nullptr), "rot_prep: the whole-row norms come together");
     I64H_CHECK_ARG(d.P && d.Q && d.positions && d.slot_ids && d.block_table && d.cache, "rot_prep: null operand");
     I64H_CHECK_ARG(d.block_size > 0 && d.max_blocks_per_seq > 0 && (d.cache_dtype == 0 || d.cache_dtype == 2), "rot_prep: bad paging or cache type");
-    const size_t lds = ((size_t)(d.heads + d.kv_heads) * (d.dim + 1) + 4) * 4;
+    const size_t lds = ((size_t)(d.heads + d.kv_heads) * (d.dim + 1) + 8 + d.rot_dims + (d.v_freq ? d.vdim : 0)) * 4;
     I64H_CHECK_ARG(lds <= 64 * 1024, "rot_prep: %d + %d heads of %d values do not fit the kernel's LDS buffer", d.heads, d.kv_heads, d.dim);
     if (d.n == 0) return 0;
     hipLaunchKernelGGL(rot_prep_kernel, dim3((unsigned)d.n), dim3(256), lds, (hipStream_t)stream, d);
@@ -916,7 +938,7 @@ int i64h_rot_post(const i64h_rot_post_args* dp, void* stream) {
     I64H_CHECK_ARG(d.heads > 0 && d.vdim > 0 && (!d.v_freq || d.vdim % 2 == 0), "rot_post: heads %d, vdim %d", d.heads, d.vdim);
     I64H_CHECK_ARG(d.O && d.positions && (d.v_freq || d.gate), "rot_post: null operand or nothing to do");
     if (d.n == 0) return 0;
-    hipLaunchKernelGGL(rot_post_kernel, dim3((unsigned)d.n), dim3(256), 0, (hipStream_t)stream, d);
+    hipLaunchKernelGGL(rot_post_kernel, dim3((unsigned)d.n), dim3(256), (size_t)d.vdim * 4, (hipStream_t)stream, d);
     I64H_CHECK_LAUNCH();
     return 0;
 }
