@@ -2,8 +2,9 @@
  * tiled Linear on the bf16 / f32 matrix cores with fused epilogues, scaled embedding, gated post-norm residual with
  * grouped RMS norm and depth mixing, latent (low-rank, shared-key) attention over a paged cache with a sliding window,
  * multi-stream and sandwich-norm residuals, causal convolutions with carried inputs, state-space / gated / gated-linear recurrences,
- * attention with a distance bias (keys as values, or separate keys and values in one cached row), expert routing with grouped
- * Linears over device-side row groups, row sampling.  A library of its own so that a process that serves such a model builds and
+ * attention with a distance bias (keys as values, or separate keys and values in one cached row), rotated attention (query / key norms,
+ * two pair layouts, rotated values, capped scores, gated heads), learned attention sinks, the gated delta rule, expert routing with
+ * grouped Linears over device-side row groups, row sampling.  A library of its own so that a process that serves such a model builds and
  * loads nothing else.
  *
  * Conventions are those of libi64hip.so (include/i64h.h): raw device pointers, caller-allocated outputs, no allocation

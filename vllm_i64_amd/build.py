@@ -3,7 +3,8 @@
 libi64hip.so        the quantized token-routed-MoE forward (include/i64h.h)
 libi64hip_dense.so  models with bf16 weights and a 32-bit residual: Linear, gated post-norm, latent attention, multi-stream
                     residual, state-space / gated recurrences, key-valued chunked attention, attention with separate keys and values,
-                    gated linear recurrence, expert routing and grouped expert Linears, sampling
+                    gated linear recurrence, rotated attention with capped scores, gated delta rule, expert routing and grouped
+                    expert Linears, sampling
                     (include/i64h_dense.h) - a library of its own, so that serving such a model builds nothing else
 """
 from __future__ import annotations

@@ -1,6 +1,7 @@
 // Kernels of libi64hip_dense.so for recurrent and hybrid layers (include/i64h_dense.h, "recurrent and hybrid layers"):
 //   embed_bigram_kernel / prev_token_kernel : token embedding + hashed bigram embedding; the previous token is per-sequence state
-//   streams_kernel        : multi-stream residual write (a result may pass a norm of its own first) + the next sublayer's weighted read
+//   streams_kernel        : multi-stream residual write (a result may pass a norm of its own first, and the result as a whole an RMS or
+//                           centred norm) + the next sublayer's weighted read
 //                           and RMS norm, one workgroup per row
 //   causal_conv_kernel / conv_carry_kernel : per-channel causal convolution over rows and carried inputs (+ silu, or added to its input);
 //                           the carry update
