@@ -594,7 +594,8 @@ __device__ __forceinline__ void rot_pair(int d, int dims, int interleaved, int& 
 // One workgroup per token, two passes: the raw queries and keys go to LDS while their squares are summed (a rotation keeps the sum of
 // squares of a pair, so the per-head sums behind the rotation are those in front of it, the rotated part times rot_mult^2); the second
 // pass norms and rotates out of LDS straight into the query rows and the cached row.
-__global__ __launch_bounds__(256) void rot_prep_kernel(const i64h_rot_prep_args p) {
+template <int NT>
+__global__ __launch_bounds__(NT) void rot_prep_kernel(const i64h_rot_prep_args p) {
     extern __shared__ float sv[];   // [heads * dim + kv_heads * dim] raw queries and keys, [heads + kv_heads] 1 / rms per head, 8 for
                                     // reductions, [rot_dims] cosines and sines of the row's angles, [vdim] those of the values' angles
     const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
@@ -612,13 +613,13 @@ __global__ __launch_bounds__(256) void rot_prep_kernel(const i64h_rot_prep_args 
     const int pos = p.positions[t];
     const float fpos = (float)pos;
     float a = 0.0f, b = 0.0f;
-    for (int c = tid; c < nq + nk; c += 256) {
+    for (int c = tid; c < nq + nk; c += NT) {
         const float x = c < nq ? q[c] : k[c - nq];
         sv[c] = x;
         if (c < nq) a += x * x;
         else b += x * x;
     }
-    for (int i = tid; i < half + vhalf; i += 256) {
+    for (int i = tid; i < half + vhalf; i += NT) {
         float sn, cs;
         if (i < half) {
             sincosf(fpos * p.inv_freq[i], &sn, &cs);
@@ -634,13 +635,16 @@ __global__ __launch_bounds__(256) void rot_prep_kernel(const i64h_rot_prep_args 
         __syncthreads();
         if (lane == 0) red[wid] = a, red[4 + wid] = b;
         __syncthreads();
-        qr = 1.0f / sqrtf((red[0] + red[1] + red[2] + red[3]) / (float)nq + p.eps);
-        kr = 1.0f / sqrtf((red[4] + red[5] + red[6] + red[7]) / (float)nk + p.eps);
+        float sa = 0.0f, sb = 0.0f;
+#pragma unroll
+        for (int w = 0; w < NT / 64; ++w) sa += red[w], sb += red[4 + w];
+        qr = 1.0f / sqrtf(sa / (float)nq + p.eps);
+        kr = 1.0f / sqrtf(sb / (float)nk + p.eps);
     }
     __syncthreads();
     if (p.head_norm) {
         const float m2 = p.rot_mult * p.rot_mult;
-        for (int h = wid; h < p.heads + p.kv_heads; h += 4) {
+        for (int h = wid; h < p.heads + p.kv_heads; h += NT / 64) {
             float s = 0.0f;
             for (int d = lane; d < dim; d += 64) {
                 const float x = sv[h * dim + d];
@@ -654,34 +658,35 @@ __global__ __launch_bounds__(256) void rot_prep_kernel(const i64h_rot_prep_args 
     float* Q = p.Q + t * p.heads * gs;
     const int64_t cr = cache_row(p.block_table, p.max_blocks_per_seq, p.block_size, p.slot_ids[t], pos);
     const int nkv = p.kv_heads * gs;
-    // every head's part of a query row and of the cached row: [vdim zeros or values | dim rotated values]
-    for (int c = tid; c < (p.heads + p.kv_heads) * gs; c += 256) {
-        const int h = c / gs, d = c % gs;
+    // every head's part of a query row and of the cached row: [vdim zeros or values | dim rotated values]; a wave takes whole heads, so
+    // that what depends on the head only is the same for all its lanes and no lane divides
+    for (int h = wid; h < p.heads + p.kv_heads; h += NT / 64) {
         const bool isq = h < p.heads;
-        float o;
-        if (d >= vd) {
-            const int e = d - vd, h0 = h * dim;      // (the keys' raw values lie behind the queries': head index heads + g)
-            const float* nw = isq ? p.q_norm_w : p.k_norm_w;
-            const float r = isq ? qr : kr;
-            const int w0 = isq ? h0 : h0 - nq;
-            auto val = [&](int idx) { return nw ? sv[h0 + idx] * r * nw[w0 + idx] : sv[h0 + idx]; };
-            if (e < p.rot_dims) {
-                int ia, ib, i;
-                bool second;
-                rot_pair(e, p.rot_dims, p.interleaved, ia, ib, i, second);
-                const float cs = rcs[i], sn = rcs[half + i];
-                const float u = val(ia), w = val(ib);
-                o = second ? w * cs + u * sn : u * cs - w * sn;
-            } else {
-                o = val(e);
-            }
-            if (p.head_norm) o *= inv[h];
-            if (isq) o *= p.scale;
-        } else if (isq) {
-            o = 0.0f;
-        } else {
-            const int g = h - p.heads;
-            if (p.v_freq) {
+        const int h0 = h * dim;                      // (the keys' raw values lie behind the queries': head index heads + g)
+        const float* nw = isq ? p.q_norm_w : p.k_norm_w;
+        const float r = isq ? qr : kr;
+        const int w0 = isq ? h0 : h0 - nq;
+        const float hn = (p.head_norm ? inv[h] : 1.0f) * (isq ? p.scale : 1.0f);
+        const int g = h - p.heads;
+        for (int d = lane; d < gs; d += 64) {
+            float o;
+            if (d >= vd) {
+                const int e = d - vd;
+                auto val = [&](int idx) { return nw ? sv[h0 + idx] * r * nw[w0 + idx] : sv[h0 + idx]; };
+                if (e < p.rot_dims) {
+                    int ia, ib, i;
+                    bool second;
+                    rot_pair(e, p.rot_dims, p.interleaved, ia, ib, i, second);
+                    const float cs = rcs[i], sn = rcs[half + i];
+                    const float u = val(ia), w = val(ib);
+                    o = second ? w * cs + u * sn : u * cs - w * sn;
+                } else {
+                    o = val(e);
+                }
+                if (p.head_norm || isq) o *= hn;
+            } else if (isq) {
+                o = 0.0f;
+            } else if (p.v_freq) {
                 int ia, ib, i;
                 bool second;
                 rot_pair(d, vd, p.interleaved, ia, ib, i, second);
@@ -691,10 +696,10 @@ __global__ __launch_bounds__(256) void rot_prep_kernel(const i64h_rot_prep_args 
             } else {
                 o = v[g * vd + d];
             }
+            if (isq) Q[h * gs + d] = o;
+            else if (p.cache_dtype == 0) ((float*)p.cache)[cr * nkv + g * gs + d] = o;
+            else ((__bf16*)p.cache)[cr * nkv + g * gs + d] = (__bf16)o;
         }
-        if (isq) Q[c] = o;
-        else if (p.cache_dtype == 0) ((float*)p.cache)[cr * nkv + c - p.heads * gs] = o;
-        else ((__bf16*)p.cache)[cr * nkv + c - p.heads * gs] = (__bf16)o;
     }
 }
 
@@ -928,7 +933,7 @@ int i64h_rot_prep(const i64h_rot_prep_args* dp, void* stream) {
     const size_t lds = ((size_t)(d.heads + d.kv_heads) * (d.dim + 1) + 8 + d.rot_dims + (d.v_freq ? d.vdim : 0)) * 4;
     I64H_CHECK_ARG(lds <= 64 * 1024, "rot_prep: %d + %d heads of %d values do not fit the kernel's LDS buffer", d.heads, d.kv_heads, d.dim);
     if (d.n == 0) return 0;
-    hipLaunchKernelGGL(rot_prep_kernel, dim3((unsigned)d.n), dim3(256), lds, (hipStream_t)stream, d);
+    hipLaunchKernelGGL(rot_prep_kernel<256>, dim3((unsigned)d.n), dim3(256), lds, (hipStream_t)stream, d);
     I64H_CHECK_LAUNCH();
     return 0;
 }
