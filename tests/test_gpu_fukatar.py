@@ -429,6 +429,37 @@ def test_latent_attention_with_learned_sinks(dev, cache_dtype, H, d, dv, r, bloc
         assert float(o[:, -1].abs().mean()) < 0.5 * float(o[:, 0].abs().mean())
 
 
+@pytest.mark.parametrize("mode", ["prompt", "decode"])
+@pytest.mark.parametrize("cache_dtype,block,T", [(torch.float32, 16, 200), (torch.bfloat16, 8, 530)])
+def test_latent_attention_one_row_stands_out(dev, mode, cache_dtype, block, T):
+    """One cached row alone lines up with the last query (every other row is orthogonal to it) - the first, one far back, those at page
+    borders, the query's own: every head returns that row's values; the sinks lie far below the score."""
+    H, d, dv, r = 3, 16, 16, 32
+    m = {"heads": H, "dim": d, "vdim": dv, "kv_rank": r, "scale": 1.0}
+    g = torch.Generator().manual_seed(T)
+    pick = torch.zeros(d, r)
+    pick[:, :d] = torch.eye(d)                                     # a head's key is the first d values of the row
+    w = {"uk": pick.repeat(H, 1).to(torch.bfloat16), "uv": (torch.randn(H * dv, r, generator=g) * r ** -0.5).to(torch.bfloat16), "dkv.norm": torch.ones(r),
+         "sink": torch.full((H,), -30.0)}
+    sel, _ = selectors({"q": H * d, "dkv": r})
+    W = {"x." + k: v for k, v in sel.items()}
+    W.update({"x.uk": w["uk"].double(), "x.uv": w["uv"].double(), "x.dkv.norm": w["dkv.norm"].double(), "x.sink": w["sink"].double(), "x.o": torch.eye(H * dv, dtype=F64)})
+    exact = cache_dtype == torch.float32
+    for target in (0, 3, block - 1, block, T - 2 * block, T - 1):
+        h = torch.zeros(T, H * d + r)
+        h[:, H * d + 1] = 1.0                                      # every row along the second direction ...
+        h[:, H * d + d:] = torch.randn(T, r - d, generator=g) * 0.25   # (... with values of its own behind the key part)
+        h[target, H * d + 1], h[target, H * d] = 0.0, 1.0          # ... but the target, along the first
+        h[T - 1, 0:H * d:d] = 6.0                                  # the last query asks along the first, in every head
+        h = h.to(torch.bfloat16).float()
+        want = R.latent_attention(W, "x.", m, 1e-6, h.double())
+        c = R.rms(h[target, H * d:].double(), 1e-6)
+        assert close(want[-1], w["uv"].double() @ c, 1e-4)         # (the premise)
+        cuts = [T] if mode == "prompt" else [T - 1, 1]
+        got = _latent_run(dev, m, w, {1: h}, {1: T}, cuts, cache_dtype, block, 1e-6, exact)
+        assert close(got[1][-1], want[-1], 2e-5 if exact else 2e-2), target
+
+
 def _delta_run(dev, m, w, h, lens, cut_sizes, eps):
     """h: slot -> [T, q | k | v | b | a | g] raw projections; convolution, gates, scan and the gated head norm through the kernels."""
     from vllm_i64_amd import ops_dense as D
