@@ -48,6 +48,17 @@ def test_registry_names_the_design():
     assert registry.architecture_of(config_of("odd")) == "Fukatar"
 
 
+def test_loader_takes_sizes_a_config_leaves_out_from_the_tensors(monkeypatch):
+    from vllm_i64_amd import fukatar, registry
+    seen = {}
+    monkeypatch.setattr(fukatar, "FukatarModel", lambda cfg, tensors, **kw: seen.update(cfg=cfg, kw=kw))
+    cfg = config_of("twotap")
+    del cfg["vocab"], cfg["width"], cfg["layers"][0]["mixer"]["right"]["conv"]
+    registry._load_fukatar(cfg, make_weights("twotap"), device="cpu", dtype="float32", max_seqs=2, max_tokens=100)
+    c = seen["cfg"]
+    assert (c.vocab, c.width, c.layers[0].mixer.right.conv) == (SHAPES["twotap"]["vocab"], SHAPES["twotap"]["width"], 2) and seen["kw"]["num_kv_blocks"] == 7
+
+
 def test_scaled_frequencies_match_the_written_out_ramp():
     from vllm_i64_amd.config import RotaryConfig
     for base, dims, sc in ((10000.0, 64, (4.0, 512, 16.0, 1.0)), (500.0, 6, (4.0, 40, 8.0, 0.5)), (77.0, 10, None), (1e6, 128, (32.0, 8192, 32.0, 1.0))):

@@ -66,6 +66,13 @@ def _load_fukatar(config: dict, tensors, *, device, dtype, max_seqs, max_tokens,
     for key, axis in (("vocab", 0), ("width", 1)):      # sizes that the file may leave to the tensors' shapes
         if key not in config and "embed" in tensors:
             config[key] = int(tensors["embed"].shape[axis])
+    layers = []
+    for i, l in enumerate(config.get("layers") or []):     # (the convolution's taps likewise, where a delta rule's entry leaves them out)
+        name = f"l{i}.mix.right.q.conv"
+        if l.get("type") == "parallel" and "conv" not in ((l.get("mixer") or {}).get("right") or {"conv": 0}) and name in tensors:
+            l = dict(l, mixer=dict(l["mixer"], right=dict(l["mixer"]["right"], conv=int(tensors[name].shape[1]))))
+        layers.append(l)
+    config["layers"] = layers
     cfg = FukatarConfig.from_dict(config)
     blocks = max(1, (int(max_tokens) + kv_block - 1) // kv_block)
     return FukatarModel(cfg, tensors, device=device, dtype=dtype, max_seqs=max_seqs, num_kv_blocks=blocks, kv_block=kv_block)
